@@ -1,0 +1,180 @@
+"""ctypes binding of lib/libxma_hip.so (declared in include/xma_hip.h).
+
+This is the only way native code is reached: there is no fallback.  If the shared object is
+missing or a kernel entry point rejects its arguments, the caller gets a RuntimeError (the
+reference raises the same type from TORCH_CHECK, xma/include/checks.h:9-15).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_void_p
+
+import torch
+
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libxma_hip.so")
+_lib: ctypes.CDLL | None = None
+
+DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+GEMM_TN, GEMM_NN, GEMM_MT = 0, 1, 2
+EPI_NONE, EPI_SWIGLU, EPI_SWIGLU_BWD = 0, 1, 2
+
+
+class GroupedGemmArgs(ctypes.Structure):
+    """struct xma_grouped_gemm_args"""
+
+    _fields_ = [
+        ("kind", c_int32),
+        ("dtype", c_int32),
+        ("epilogue", c_int32),
+        ("num_experts", c_int32),
+        ("rows", c_int64),
+        ("n", c_int64),
+        ("k", c_int64),
+        ("a", c_void_p),
+        ("lda", c_int64),
+        ("b", c_void_p),
+        ("ldb", c_int64),
+        ("b_expert_stride", c_int64),
+        ("c", c_void_p),
+        ("ldc", c_int64),
+        ("c_expert_stride", c_int64),
+        ("aux", c_void_p),
+        ("ld_aux", c_int64),
+        ("expert_offsets", c_void_p),
+        ("in_index", c_void_p),
+        ("out_index", c_void_p),
+        ("idx_is_i64", c_int32),
+        ("in_fan_out", c_int32),
+        ("workspace", c_void_p),
+        ("workspace_bytes", c_int64),
+    ]
+
+
+# name -> (restype, argtypes); must list every symbol include/xma_hip.h declares
+PROTOTYPES: dict[str, tuple] = {
+    "xma_last_error": (c_char_p, []),
+    "xma_version": (c_char_p, []),
+    "xma_target_arch": (c_char_p, []),
+    "xma_continuous_count": (c_int, [c_void_p, c_int, c_int64, c_int32, c_void_p, c_void_p]),
+    "xma_route_workspace_bytes": (c_int64, [c_int64, c_int32]),
+    "xma_route_build": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_void_p],
+    ),
+    "xma_topk_softmax": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int32, c_int32, c_int64, c_void_p, c_void_p, c_int, c_void_p],
+    ),
+    "xma_topk_softmax_bwd": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int64, c_int32, c_int32, c_void_p, c_int64, c_void_p],
+    ),
+    "xma_gather_rows": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int64, c_int, c_int32, c_void_p, c_void_p],
+    ),
+    "xma_scatter_rows": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int64, c_int, c_void_p],
+    ),
+    "xma_combine_topk": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int, c_void_p],
+    ),
+    "xma_gate_grad": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int32, c_int64, c_int, c_void_p],
+    ),
+    "xma_swiglu_forward": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p],
+    ),
+    "xma_swiglu_backward": (
+        c_int,
+        [
+            c_void_p,
+            c_int64,
+            c_void_p,
+            c_int64,
+            c_void_p,
+            c_int64,
+            c_void_p,
+            c_int64,
+            c_void_p,
+            c_int64,
+            c_int64,
+            c_int64,
+            c_int,
+            c_void_p,
+        ],
+    ),
+    "xma_grouped_gemm_workspace_bytes": (c_int64, [c_int32, c_int64]),
+    "xma_grouped_gemm": (c_int, [POINTER(GroupedGemmArgs), c_void_p]),
+}
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def is_built() -> bool:
+    return os.path.exists(_LIB_PATH)
+
+
+def load() -> ctypes.CDLL:
+    """Load the kernel library once; raises if it has not been built."""
+
+    global _lib
+    if _lib is None:
+        if not is_built():
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: build the HIP kernels with "
+                "`python -m flash_model_architectures_amd.build` (needs hipcc); there is no fallback path"
+            )
+        lib = ctypes.CDLL(_LIB_PATH)
+        for name, (restype, argtypes) in PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().xma_last_error().decode()
+
+
+def call(name: str, *args) -> None:
+    """Invoke an int-returning entry point and turn a non-zero status into RuntimeError."""
+
+    status = getattr(load(), name)(*args)
+    if status != 0:
+        raise RuntimeError(f"{name} failed: {last_error()}")
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    try:
+        return DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}: expected float32, float16 or bfloat16") from None
+
+
+def require_device(*tensors: torch.Tensor | None) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "the HIP kernels need tensors on a ROCm device (got a tensor on "
+                f"{t.device}); there is no CPU path in this package"
+            )
+
+
+def ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def stream() -> int:
+    return torch.cuda.current_stream().cuda_stream

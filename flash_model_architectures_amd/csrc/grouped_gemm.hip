@@ -1,0 +1,717 @@
+// Ragged (per-expert) GEMM for gfx950 with MFMA and fp32 accumulation.
+//
+// One kernel body serves the three operand layouts of the MoE layer; they differ only in how a
+// tile is fetched from HBM:
+//   TN  C[p, n] = sum_k A[row(p), k] * W[e][n, k]     forward projections (optional row gather on A)
+//   NN  C[p, n] = sum_k A[p, k]      * W[e][k, n]     input gradients
+//   MT  C[e][i, j] = sum_p A[p, i] * B[row(p), j]     weight gradients (reduction over routed rows)
+// Inside LDS both operands always look the same: [tile rows][BK] with the reduction index
+// contiguous, 128 bytes per row, the eight 16-byte chunks of a row XOR-swizzled by the row
+// number.  Operands whose reduction index is strided in HBM (W in NN, both in MT) are fetched as
+// PV x PV element blocks (PV = elements per 16 bytes), transposed in registers, and written to
+// LDS as whole chunks.  The MFMA loop reads 16-byte fragments, multiplies 32x32 sub-tiles, and
+// the epilogue stages the tile in LDS again so that HBM sees full 16-byte row-wise stores
+// (optionally fused with SwiGLU forward / backward, row scatter).
+//
+// Work-group -> tile mapping: a prologue kernel expands the expert offsets into a list of row
+// tiles (expert, first row), so ragged and empty groups cost nothing; the main kernel renumbers
+// work-groups so that each of the 8 XCDs (private L2 each) owns a contiguous range of tiles, and
+// walks tiles in bands of 4 row tiles x all column tiles to reuse both panels from L2.
+#include "common.h"
+
+namespace xma {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+constexpr int kNumXcd = 8;
+constexpr int kBandTiles = 4;  // row tiles per band of the tile walk
+
+// ---- per-dtype tile configuration -----------------------------------------------------------
+template <typename T>
+struct TileCfg {  // 16-bit element types
+    static constexpr int BM = 256, BN = 256, BK = 64, THREADS = 512, WAVES_M = 2, WAVES_N = 4;
+};
+template <>
+struct TileCfg<float> {
+    static constexpr int BM = 128, BN = 128, BK = 32, THREADS = 256, WAVES_M = 2, WAVES_N = 2;
+};
+
+constexpr int kLdsRowBytes = 128;  // BK * sizeof(T) for every configuration
+constexpr int kChunksPerRow = 8;
+
+__device__ __forceinline__ int swizzle_of_row(int row) { return ((row >> 1) ^ (row >> 4)) & 7; }
+__device__ __forceinline__ int lds_chunk_offset(int row, int chunk) {
+    return row * kLdsRowBytes + ((chunk ^ swizzle_of_row(row)) << 4);
+}
+
+// ---- MFMA wrappers: acc(32x32) += X(32 rows x kslice) * Y(32 cols x kslice)^T ----------------------
+template <typename T>
+struct Mma;
+template <>
+struct Mma<bf16_t> {
+    __device__ static __forceinline__ void run(const uint4& x, const uint4& y, f32x16_t& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, x), __builtin_bit_cast(bf16x8_t, y),
+                                                      acc, 0, 0, 0);
+    }
+};
+template <>
+struct Mma<f16_t> {
+    __device__ static __forceinline__ void run(const uint4& x, const uint4& y, f32x16_t& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, x), __builtin_bit_cast(f16x8_t, y),
+                                                     acc, 0, 0, 0);
+    }
+};
+template <>
+struct Mma<float> {
+    // a 16-byte fragment holds 4 reduction steps per lane half; one 32x32x2 MFMA per component
+    __device__ static __forceinline__ void run(const uint4& x, const uint4& y, f32x16_t& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.x), __uint_as_float(y.x), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.y), __uint_as_float(y.y), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.z), __uint_as_float(y.z), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.w), __uint_as_float(y.w), acc, 0, 0, 0);
+    }
+};
+
+// ---- register transposes of a PV x PV block ---------------------------------------------------
+// in[r] = PV consecutive elements of block row r; out[c] = the PV elements of block column c.
+__device__ __forceinline__ uint32_t pack_lo(uint32_t a, uint32_t b) { return (a & 0xffffu) | (b << 16); }
+__device__ __forceinline__ uint32_t pack_hi(uint32_t a, uint32_t b) { return (a >> 16) | (b & 0xffff0000u); }
+
+template <int PV>
+__device__ __forceinline__ void transpose_block(const uint4 (&in)[PV], uint4 (&out)[PV]);
+
+template <>
+__device__ __forceinline__ void transpose_block<8>(const uint4 (&in)[8], uint4 (&out)[8]) {
+#define XMA_T16(J, D)                                                                                       \
+    out[2 * J] = make_uint4(pack_lo(in[0].D, in[1].D), pack_lo(in[2].D, in[3].D), pack_lo(in[4].D, in[5].D), \
+                            pack_lo(in[6].D, in[7].D));                                                     \
+    out[2 * J + 1] = make_uint4(pack_hi(in[0].D, in[1].D), pack_hi(in[2].D, in[3].D), pack_hi(in[4].D, in[5].D), \
+                                pack_hi(in[6].D, in[7].D));
+    XMA_T16(0, x)
+    XMA_T16(1, y)
+    XMA_T16(2, z)
+    XMA_T16(3, w)
+#undef XMA_T16
+}
+
+template <>
+__device__ __forceinline__ void transpose_block<4>(const uint4 (&in)[4], uint4 (&out)[4]) {
+    out[0] = make_uint4(in[0].x, in[1].x, in[2].x, in[3].x);
+    out[1] = make_uint4(in[0].y, in[1].y, in[2].y, in[3].y);
+    out[2] = make_uint4(in[0].z, in[1].z, in[2].z, in[3].z);
+    out[3] = make_uint4(in[0].w, in[1].w, in[2].w, in[3].w);
+}
+
+__device__ __forceinline__ uint4 load16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ uint4 zero16() { return make_uint4(0u, 0u, 0u, 0u); }
+
+// ---- tile loaders -----------------------------------------------------------------------------
+// DirectLoader: the operand's reduction index is contiguous in HBM.  NT threads starting at
+// thread T0 copy R rows x 8 chunks per stage; each thread keeps its chunk column and walks rows.
+template <typename T, int R, int NT, int T0>
+struct DirectLoader {
+    static constexpr int PV = Elem<T>::kPerVec;
+    static constexpr int ITEMS = R * kChunksPerRow / NT;
+    static constexpr int ROW_STEP = NT / kChunksPerRow;
+    const T* row_ptr[ITEMS];  // points at the thread's chunk in reduction step 0; nullptr = masked row
+    int chunk;
+    int row0;
+    bool active;
+
+    template <typename RowFn>
+    __device__ __forceinline__ void init(int tid, RowFn row_fn) {
+        const int lt = tid - T0;
+        active = lt >= 0 && lt < NT;
+        chunk = lt & (kChunksPerRow - 1);
+        row0 = lt / kChunksPerRow;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const T* p = active ? row_fn(row0 + i * ROW_STEP) : nullptr;
+            row_ptr[i] = p ? p + chunk * PV : nullptr;
+        }
+    }
+    // k0: first reduction index of the stage, klen: total reduction length
+    template <int NV>
+    __device__ __forceinline__ void load(uint4 (&v)[NV], int64_t k0, int64_t klen) const {
+        static_assert(NV >= ITEMS, "staging registers");
+        if (!active) return;
+        const bool k_ok = k0 + chunk * PV < klen;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) v[i] = (row_ptr[i] && k_ok) ? load16(row_ptr[i] + k0) : zero16();
+    }
+    template <int NV>
+    __device__ __forceinline__ void store(const uint4 (&v)[NV], char* lds) const {
+        if (!active) return;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const int row = row0 + i * ROW_STEP;
+            *reinterpret_cast<uint4*>(lds + lds_chunk_offset(row, chunk)) = v[i];
+        }
+    }
+};
+
+// TransLoader: the operand's tile-row index is contiguous in HBM and the reduction index walks
+// HBM rows.  Each of NT = 8 * R / PV threads fetches PV reduction rows x PV tile rows, transposes
+// the block in registers and writes PV chunks.
+template <typename T, int R, int NT, int T0>
+struct TransLoader {
+    static constexpr int PV = Elem<T>::kPerVec;
+    static constexpr int TCOLS = R / PV;
+    static_assert(NT == kChunksPerRow * TCOLS, "one PV x PV block per thread");
+    int tcol, tk;
+    bool active;
+
+    __device__ __forceinline__ void init(int tid) {
+        const int lt = tid - T0;
+        active = lt >= 0 && lt < NT;
+        tcol = lt % TCOLS;
+        tk = lt / TCOLS;
+    }
+    // ptr_fn(r) returns the HBM address of reduction row (tk*PV + r) of this stage at this thread's
+    // PV tile rows, or nullptr when that row / those tile rows are out of range
+    template <int NV, typename PtrFn>
+    __device__ __forceinline__ void load(uint4 (&v)[NV], PtrFn ptr_fn) const {
+        static_assert(NV >= PV, "staging registers");
+        if (!active) return;
+#pragma unroll
+        for (int r = 0; r < PV; ++r) {
+            const T* p = ptr_fn(tk * PV + r, tcol * PV);
+            v[r] = p ? load16(p) : zero16();
+        }
+    }
+    template <int NV>
+    __device__ __forceinline__ void store(const uint4 (&v)[NV], char* lds) const {
+        if (!active) return;
+        uint4 in[PV], o[PV];
+#pragma unroll
+        for (int r = 0; r < PV; ++r) in[r] = v[r];
+        transpose_block<PV>(in, o);
+#pragma unroll
+        for (int c = 0; c < PV; ++c) *reinterpret_cast<uint4*>(lds + lds_chunk_offset(tcol * PV + c, tk)) = o[c];
+    }
+};
+
+// ---- kernel arguments -----------------------------------------------------------------------------
+struct GemmParams {
+    const void* a;
+    const void* b;
+    void* c;
+    void* aux;
+    const int32_t* offsets;
+    const void* in_index;
+    const void* out_index;
+    const int32_t* tile_expert;  // [row tiles] expert of each row tile (TN/NN)
+    const int32_t* tile_row0;    // [row tiles] first grouped row of each row tile
+    const int32_t* tile_count;   // [1] number of row tiles actually present
+    int64_t lda, ldb, ldc, ld_aux, b_expert_stride, c_expert_stride;
+    int64_t n, k;
+    int32_t num_experts, in_fan_out, idx_is_i64;
+    int32_t row_tiles_max;  // upper bound used for the grid (TN/NN); MT: row tiles per expert
+    int32_t col_tiles;
+};
+
+// routed row p -> source row of the gathered operand (indices are < 2^31, so divide in 32 bits)
+__device__ __forceinline__ int64_t source_row(const GemmParams& P, int64_t p) {
+    return (int64_t)((uint32_t)load_index(P.in_index, P.idx_is_i64, p) / (uint32_t)P.in_fan_out);
+}
+
+// Row-tile list for the row-grouped kinds: expert e owns ceil(count_e / BM) consecutive tiles.
+__global__ __launch_bounds__(1024) void build_row_tiles_kernel(const int32_t* __restrict__ offsets, int E, int BM,
+                                                                int32_t* __restrict__ tile_expert,
+                                                                int32_t* __restrict__ tile_row0,
+                                                                int32_t* __restrict__ tile_count) {
+    __shared__ int32_t part[1024];
+    const int per = (E + 1023) / 1024;
+    const int e0 = threadIdx.x * per;
+    int32_t s = 0;
+    for (int i = 0; i < per; ++i) {
+        const int e = e0 + i;
+        if (e < E) s += (offsets[e + 1] - offsets[e] + BM - 1) / BM;
+    }
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        const int32_t v = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+        __syncthreads();
+        part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    int32_t t = part[threadIdx.x] - s;
+    for (int i = 0; i < per; ++i) {
+        const int e = e0 + i;
+        if (e < E) {
+            const int32_t begin = offsets[e], end = offsets[e + 1];
+            for (int32_t r = begin; r < end; r += BM) {
+                tile_expert[t] = e;
+                tile_row0[t] = r;
+                ++t;
+            }
+        }
+    }
+    if (threadIdx.x == 1023) tile_count[0] = part[1023];
+}
+
+template <typename T, int KIND, int EPI>
+__global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const GemmParams P) {
+    using Cfg = TileCfg<T>;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, THREADS = Cfg::THREADS;
+    constexpr int PV = Elem<T>::kPerVec;
+    constexpr int WM = BM / Cfg::WAVES_M, WN = BN / Cfg::WAVES_N;
+    constexpr int MI = WM / 32, NI = WN / 32;
+    constexpr int STAGE_BYTES = (BM + BN) * kLdsRowBytes;
+    constexpr int C_ROW_BYTES = BN * (int)sizeof(T) + 16;
+    // column tile width in units of output columns: the SwiGLU epilogue packs BN/2 `up` and BN/2
+    // `gate` columns into one tile
+    constexpr int BN_OUT = EPI == XMA_EPI_SWIGLU ? BN / 2 : BN;
+    static_assert(BK * sizeof(T) == kLdsRowBytes, "LDS rows are 128 bytes");
+
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm0 = (wave / Cfg::WAVES_N) * WM;
+    const int wn0 = (wave % Cfg::WAVES_N) * WN;
+
+    // ---- which tile ----
+    // work-groups are dealt round-robin to the XCDs; give each XCD a contiguous range of tiles
+    const int nwg = gridDim.x;  // multiple of kNumXcd
+    const int pid = (blockIdx.x % kNumXcd) * (nwg / kNumXcd) + blockIdx.x / kNumXcd;
+    const int row_tiles = KIND == XMA_GEMM_MT ? P.row_tiles_max * P.num_experts : P.tile_count[0];
+    const int col_tiles = P.col_tiles;
+    const int band = pid / (kBandTiles * col_tiles);
+    const int band_first = band * kBandTiles;
+    if (band_first >= row_tiles) return;
+    const int band_rows = row_tiles - band_first < kBandTiles ? row_tiles - band_first : kBandTiles;
+    const int in_band = pid - band * (kBandTiles * col_tiles);
+    const int row_tile = band_first + in_band % band_rows;
+    const int col_tile = in_band / band_rows;
+    if (col_tile >= col_tiles) return;
+
+    const T* A = reinterpret_cast<const T*>(P.a);
+    const T* B = reinterpret_cast<const T*>(P.b);
+
+    int expert;
+    int64_t m_begin, m_end;      // grouped rows covered by this tile (TN/NN) or reduced over (MT)
+    int64_t tile_i0 = 0;         // MT: first row of C[e] in this tile
+    int64_t n0;                  // first output column (TN/NN) / first column of C[e] (MT)
+    int64_t red_len;             // reduction length
+    if constexpr (KIND == XMA_GEMM_MT) {
+        expert = row_tile / P.row_tiles_max;
+        tile_i0 = (int64_t)(row_tile % P.row_tiles_max) * BM;
+        m_begin = P.offsets[expert];
+        m_end = P.offsets[expert + 1];
+        red_len = m_end - m_begin;
+        n0 = (int64_t)col_tile * BN;
+    } else {
+        expert = P.tile_expert[row_tile];
+        m_begin = P.tile_row0[row_tile];
+        const int64_t e_end = P.offsets[expert + 1];
+        m_end = m_begin + BM < e_end ? m_begin + BM : e_end;
+        red_len = P.k;
+        n0 = (int64_t)col_tile * BN_OUT;
+    }
+
+    // ---- loaders ----
+    constexpr bool A_TRANS = KIND == XMA_GEMM_MT;
+    constexpr bool B_TRANS = KIND != XMA_GEMM_TN;
+    constexpr bool SPLIT = sizeof(T) == 2 && (A_TRANS || B_TRANS);  // halves of the block serve one operand each
+    constexpr int NT_HALF = THREADS / 2;
+    // thread ranges: (count, first thread) per operand
+    constexpr int A_NT = SPLIT ? NT_HALF : THREADS;
+    constexpr int A_T0 = (SPLIT && KIND == XMA_GEMM_NN) ? NT_HALF : 0;
+    constexpr int B_NT = SPLIT ? NT_HALF : THREADS;
+    constexpr int B_T0 = (SPLIT && KIND == XMA_GEMM_MT) ? NT_HALF : 0;
+
+    DirectLoader<T, BM, A_NT, A_T0> a_direct;
+    TransLoader<T, BM, kChunksPerRow * BM / PV, A_T0> a_trans;
+    DirectLoader<T, BN, B_NT, B_T0> b_direct;
+    TransLoader<T, BN, kChunksPerRow * BN / PV, B_T0> b_trans;
+    // Staging registers between HBM and LDS.  When the block is split, a thread serves one operand
+    // only, so both loaders share one register set.
+    constexpr int A_REGS = A_TRANS ? PV : BM * kChunksPerRow / A_NT;
+    constexpr int B_REGS = B_TRANS ? PV : BN * kChunksPerRow / B_NT;
+    uint4 st_a[A_REGS > B_REGS || !SPLIT ? A_REGS : B_REGS];
+    uint4 st_b_own[SPLIT ? 1 : B_REGS];
+    auto& st_b = [&]() -> auto& {
+        if constexpr (SPLIT)
+            return st_a;
+        else
+            return st_b_own;
+    }();
+    static_assert(!A_TRANS || kChunksPerRow * BM / PV == A_NT, "A transposing loader thread count");
+    static_assert(!B_TRANS || kChunksPerRow * BN / PV == B_NT, "B transposing loader thread count");
+
+    const T* Wexp = B + (KIND == XMA_GEMM_MT ? 0 : (int64_t)expert * P.b_expert_stride);
+
+    if constexpr (!A_TRANS) {
+        a_direct.init(tid, [&](int r) -> const T* {
+            const int64_t p = m_begin + r;
+            if (p >= m_end) return nullptr;
+            const int64_t src = P.in_index ? source_row(P, p) : p;
+            return A + src * P.lda;
+        });
+    } else {
+        a_trans.init(tid);
+    }
+    if constexpr (!B_TRANS) {
+        b_direct.init(tid, [&](int r) -> const T* {
+            int64_t n;
+            if constexpr (EPI == XMA_EPI_SWIGLU) {
+                const int64_t half = P.n / 2;
+                const int64_t j = n0 + (r % BN_OUT);
+                if (j >= half) return nullptr;
+                n = r < BN_OUT ? j : half + j;
+            } else {
+                n = n0 + r;
+                if (n >= P.n) return nullptr;
+            }
+            return Wexp + n * P.ldb;
+        });
+    } else {
+        b_trans.init(tid);
+    }
+
+    auto load_stage = [&](int64_t k0) {
+        if constexpr (!A_TRANS) {
+            a_direct.load(st_a, k0, red_len);
+        } else {
+            a_trans.load(st_a, [&](int r, int col) -> const T* {
+                const int64_t p = m_begin + k0 + r;
+                const int64_t i = tile_i0 + col;
+                return (p < m_end && i < P.n) ? A + p * P.lda + i : nullptr;
+            });
+        }
+        if constexpr (!B_TRANS) {
+            b_direct.load(st_b, k0, red_len);
+        } else if constexpr (KIND == XMA_GEMM_NN) {
+            b_trans.load(st_b, [&](int r, int col) -> const T* {
+                const int64_t kk = k0 + r;
+                const int64_t n = n0 + col;
+                return (kk < P.k && n < P.n) ? Wexp + kk * P.ldb + n : nullptr;
+            });
+        } else {
+            b_trans.load(st_b, [&](int r, int col) -> const T* {
+                const int64_t p = m_begin + k0 + r;
+                const int64_t j = n0 + col;
+                if (p >= m_end || j >= P.k) return nullptr;
+                const int64_t src = P.in_index ? source_row(P, p) : p;
+                return B + src * P.ldb + j;
+            });
+        }
+    };
+    auto store_stage = [&](int buf) {
+        char* base = lds + buf * STAGE_BYTES;
+        if constexpr (!A_TRANS)
+            a_direct.store(st_a, base);
+        else
+            a_trans.store(st_a, base);
+        if constexpr (!B_TRANS)
+            b_direct.store(st_b, base + BM * kLdsRowBytes);
+        else
+            b_trans.store(st_b, base + BM * kLdsRowBytes);
+    };
+
+    // ---- accumulators and fragment addressing ----
+    f32x16_t acc[MI][NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
+
+    const int frag_row = lane & 31;
+    const int frag_half = lane >> 5;
+    int a_off[MI], a_sw[MI], b_off[NI], b_sw[NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+        const int row = wm0 + mi * 32 + frag_row;
+        a_off[mi] = row * kLdsRowBytes;
+        a_sw[mi] = swizzle_of_row(row);
+    }
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+        const int row = wn0 + ni * 32 + frag_row;
+        b_off[ni] = BM * kLdsRowBytes + row * kLdsRowBytes;
+        b_sw[ni] = swizzle_of_row(row);
+    }
+
+    const int64_t num_stages = (red_len + BK - 1) / BK;
+    if (num_stages > 0) {
+        load_stage(0);
+        store_stage(0);
+    }
+    __syncthreads();
+    for (int64_t s = 0; s < num_stages; ++s) {
+        const bool more = s + 1 < num_stages;
+        if (more) load_stage((s + 1) * BK);
+        const char* base = lds + (int)(s & 1) * STAGE_BYTES;
+#pragma unroll
+        for (int kk = 0; kk < kChunksPerRow / 2; ++kk) {
+            const int chunk = 2 * kk + frag_half;
+            uint4 af[MI], bfr[NI];
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+                af[mi] = *reinterpret_cast<const uint4*>(base + a_off[mi] + ((chunk ^ a_sw[mi]) << 4));
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+                bfr[ni] = *reinterpret_cast<const uint4*>(base + b_off[ni] + ((chunk ^ b_sw[ni]) << 4));
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) Mma<T>::run(bfr[ni], af[mi], acc[mi][ni]);
+        }
+        if (more) store_stage((int)((s + 1) & 1));
+        __syncthreads();
+    }
+
+    // ---- epilogue: registers -> LDS tile [BM][BN] -> HBM ----
+    // MFMA result element r of lane l: tile column = 8*(r/4) + 4*(l/32) + r%4 (+32*ni), tile row = l%32 (+32*mi)
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+        const int row = wm0 + mi * 32 + frag_row;
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int col = wn0 + ni * 32 + 8 * g + 4 * frag_half;
+                char* dst = lds + row * C_ROW_BYTES + col * (int)sizeof(T);
+                const float f[4] = {acc[mi][ni][4 * g], acc[mi][ni][4 * g + 1], acc[mi][ni][4 * g + 2],
+                                    acc[mi][ni][4 * g + 3]};
+                if constexpr (sizeof(T) == 4) {
+                    *reinterpret_cast<uint4*>(dst) = Elem<float>::pack(f);
+                } else {
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(Elem<T>::pack2(f[0], f[1]), Elem<T>::pack2(f[2], f[3]));
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    constexpr int C_CHUNKS = BN / PV;          // 16-byte chunks per tile row
+    constexpr int ROWS_PER_PASS = THREADS / C_CHUNKS;
+    const int cc = tid % C_CHUNKS;
+    T* C = reinterpret_cast<T*>(P.c);
+#pragma unroll 1
+    for (int r = tid / C_CHUNKS; r < BM; r += ROWS_PER_PASS) {
+        const char* src = lds + r * C_ROW_BYTES;
+        if constexpr (KIND == XMA_GEMM_MT) {
+            const int64_t i = tile_i0 + r, j = n0 + cc * PV;
+            if (i < P.n && j < P.k)
+                *reinterpret_cast<uint4*>(C + (int64_t)expert * P.c_expert_stride + i * P.ldc + j) =
+                    *reinterpret_cast<const uint4*>(src + cc * 16);
+        } else {
+            const int64_t p = m_begin + r;
+            if (p >= m_end) break;
+            const int64_t orow = P.out_index ? load_index(P.out_index, P.idx_is_i64, p) : p;
+            if constexpr (EPI == XMA_EPI_NONE) {
+                const int64_t n = n0 + cc * PV;
+                if (n < P.n) *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = *reinterpret_cast<const uint4*>(src + cc * 16);
+            } else if constexpr (EPI == XMA_EPI_SWIGLU) {
+                constexpr int HALF_CHUNKS = C_CHUNKS / 2;
+                const int64_t half = P.n / 2;
+                const int64_t j = n0 + (cc % HALF_CHUNKS) * PV;
+                if (j < half) {
+                    if (P.aux) {
+                        T* h = reinterpret_cast<T*>(P.aux) + p * P.ld_aux;
+                        *reinterpret_cast<uint4*>(h + (cc < HALF_CHUNKS ? j : half + j)) =
+                            *reinterpret_cast<const uint4*>(src + cc * 16);
+                    }
+                    if (cc < HALF_CHUNKS) {
+                        float u[PV], g[PV], o[PV];
+                        Elem<T>::unpack(*reinterpret_cast<const uint4*>(src + cc * 16), u);
+                        Elem<T>::unpack(*reinterpret_cast<const uint4*>(src + (cc + HALF_CHUNKS) * 16), g);
+#pragma unroll
+                        for (int q = 0; q < PV; ++q) o[q] = u[q] * (g[q] * sigmoid_f32(g[q]));
+                        *reinterpret_cast<uint4*>(C + orow * P.ldc + j) = Elem<T>::pack(o);
+                    }
+                }
+            } else {  // XMA_EPI_SWIGLU_BWD
+                const int64_t n = n0 + cc * PV;
+                if (n < P.n) {
+                    const T* h = reinterpret_cast<const T*>(P.aux) + p * P.ld_aux;
+                    float u[PV], g[PV], d[PV], du[PV], dg[PV];
+                    Elem<T>::unpack(load16(h + n), u);
+                    Elem<T>::unpack(load16(h + P.n + n), g);
+                    Elem<T>::unpack(*reinterpret_cast<const uint4*>(src + cc * 16), d);
+#pragma unroll
+                    for (int q = 0; q < PV; ++q) {
+                        const float sg = sigmoid_f32(g[q]);
+                        dg[q] = d[q] * u[q] * (sg + g[q] * sg * (1.0f - sg));
+                        du[q] = d[q] * g[q] * sg;
+                    }
+                    *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = Elem<T>::pack(du);
+                    *reinterpret_cast<uint4*>(C + orow * P.ldc + P.n + n) = Elem<T>::pack(dg);
+                }
+            }
+        }
+    }
+}
+
+template <typename T>
+constexpr int lds_bytes() {
+    using Cfg = TileCfg<T>;
+    constexpr int stages = 2 * (Cfg::BM + Cfg::BN) * kLdsRowBytes;
+    constexpr int ctile = Cfg::BM * (Cfg::BN * (int)sizeof(T) + 16);
+    return stages > ctile ? stages : ctile;
+}
+
+static int64_t max_row_tiles(int64_t rows, int E, int BM) { return rows / BM + E; }
+
+template <typename T, int KIND, int EPI>
+static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
+    using Cfg = TileCfg<T>;
+    constexpr int PV = Elem<T>::kPerVec;
+    GemmParams P;
+    P.a = a.a;
+    P.b = a.b;
+    P.c = a.c;
+    P.aux = a.aux;
+    P.offsets = a.expert_offsets;
+    P.in_index = a.in_index;
+    P.out_index = a.out_index;
+    P.lda = a.lda;
+    P.ldb = a.ldb;
+    P.ldc = a.ldc;
+    P.ld_aux = a.ld_aux;
+    P.b_expert_stride = a.b_expert_stride;
+    P.c_expert_stride = a.c_expert_stride;
+    P.n = a.n;
+    P.k = a.k;
+    P.num_experts = a.num_experts;
+    P.in_fan_out = a.in_fan_out > 0 ? a.in_fan_out : 1;
+    P.idx_is_i64 = a.idx_is_i64;
+    P.tile_expert = nullptr;
+    P.tile_row0 = nullptr;
+    P.tile_count = nullptr;
+
+    int64_t tiles;
+    if (KIND == XMA_GEMM_MT) {
+        P.row_tiles_max = (int32_t)ceil_div(a.n, Cfg::BM);
+        P.col_tiles = (int32_t)ceil_div(a.k, Cfg::BN);
+        tiles = ceil_div((int64_t)P.row_tiles_max * a.num_experts, kBandTiles) * kBandTiles * P.col_tiles;
+    } else {
+        const int64_t rt = max_row_tiles(a.rows, a.num_experts, Cfg::BM);
+        int32_t* ws = reinterpret_cast<int32_t*>(a.workspace);
+        P.tile_count = ws;
+        P.tile_expert = ws + 4;
+        P.tile_row0 = ws + 4 + rt;
+        P.row_tiles_max = (int32_t)rt;
+        const int bn_out = EPI == XMA_EPI_SWIGLU ? Cfg::BN / 2 : Cfg::BN;
+        const int64_t n_out = EPI == XMA_EPI_SWIGLU ? a.n / 2 : a.n;
+        P.col_tiles = (int32_t)ceil_div(n_out, bn_out);
+        // whole bands of kBandTiles row tiles, so that every present row tile has a work-group
+        tiles = ceil_div(rt, kBandTiles) * kBandTiles * P.col_tiles;
+        hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(1024), 0, stream, a.expert_offsets, a.num_experts,
+                           Cfg::BM, ws + 4, ws + 4 + rt, ws);
+    }
+    const int64_t grid = ceil_div(tiles, kNumXcd) * kNumXcd;
+    XMA_REQUIRE(grid < ((int64_t)1 << 31), "xma_grouped_gemm: %lld tiles exceed the grid limit", (long long)grid);
+    (void)PV;
+    auto kernel = grouped_gemm_kernel<T, KIND, EPI>;
+    static bool attr_set = false;  // per instantiation
+    if (!attr_set) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<T>());
+        if (err != hipSuccess) {
+            set_error("xma_grouped_gemm: cannot reserve %d bytes of LDS: %s", lds_bytes<T>(), hipGetErrorString(err));
+            return 2;
+        }
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(Cfg::THREADS), lds_bytes<T>(), stream, P);
+    return check_launch("xma_grouped_gemm");
+}
+
+template <typename T>
+static int dispatch_kind(const xma_grouped_gemm_args& a, hipStream_t stream) {
+    switch (a.kind) {
+        case XMA_GEMM_TN:
+            if (a.epilogue == XMA_EPI_SWIGLU) return launch<T, XMA_GEMM_TN, XMA_EPI_SWIGLU>(a, stream);
+            return launch<T, XMA_GEMM_TN, XMA_EPI_NONE>(a, stream);
+        case XMA_GEMM_NN:
+            if (a.epilogue == XMA_EPI_SWIGLU_BWD) return launch<T, XMA_GEMM_NN, XMA_EPI_SWIGLU_BWD>(a, stream);
+            return launch<T, XMA_GEMM_NN, XMA_EPI_NONE>(a, stream);
+        default:
+            return launch<T, XMA_GEMM_MT, XMA_EPI_NONE>(a, stream);
+    }
+}
+
+static int largest_bm() { return TileCfg<bf16_t>::BM > TileCfg<float>::BM ? TileCfg<bf16_t>::BM : TileCfg<float>::BM; }
+static int smallest_bm() { return TileCfg<bf16_t>::BM < TileCfg<float>::BM ? TileCfg<bf16_t>::BM : TileCfg<float>::BM; }
+
+}  // namespace xma
+
+using namespace xma;
+
+extern "C" {
+
+int64_t xma_grouped_gemm_workspace_bytes(int32_t num_experts, int64_t rows) {
+    if (num_experts < 1 || rows < 0) return -1;
+    (void)largest_bm();
+    const int64_t rt = max_row_tiles(rows, num_experts, smallest_bm());
+    return (4 + 2 * rt) * (int64_t)sizeof(int32_t);
+}
+
+int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
+    XMA_REQUIRE(args != nullptr, "xma_grouped_gemm: null args");
+    const xma_grouped_gemm_args& a = *args;
+    XMA_REQUIRE(valid_dtype(a.dtype), "xma_grouped_gemm: bad dtype %d", a.dtype);
+    XMA_REQUIRE(a.kind >= XMA_GEMM_TN && a.kind <= XMA_GEMM_MT, "xma_grouped_gemm: bad kind %d", a.kind);
+    XMA_REQUIRE(a.num_experts >= 1 && a.num_experts <= 16384, "xma_grouped_gemm: num_experts=%d outside [1, 16384]",
+                a.num_experts);
+    XMA_REQUIRE(a.rows >= 0 && a.rows < ((int64_t)1 << 31) && a.n >= 0 && a.k >= 0, "xma_grouped_gemm: bad sizes");
+    XMA_REQUIRE(a.expert_offsets != nullptr, "xma_grouped_gemm: expert_offsets is null");
+    const int pv = a.dtype == XMA_F32 ? 4 : 8;
+    XMA_REQUIRE(a.n % pv == 0 && a.k % pv == 0, "xma_grouped_gemm: n=%lld and k=%lld must be multiples of %d",
+                (long long)a.n, (long long)a.k, pv);
+    XMA_REQUIRE(a.lda % pv == 0 && a.ldb % pv == 0 && a.ldc % pv == 0 && a.b_expert_stride % pv == 0 &&
+                    a.c_expert_stride % pv == 0 && a.ld_aux % pv == 0,
+                "xma_grouped_gemm: strides must keep rows 16-byte aligned");
+    XMA_REQUIRE(aligned16(a.a) && aligned16(a.b) && aligned16(a.c) && aligned16(a.aux),
+                "xma_grouped_gemm: operands must be 16-byte aligned");
+    const bool mt = a.kind == XMA_GEMM_MT;
+    if (mt) {
+        XMA_REQUIRE(a.epilogue == XMA_EPI_NONE, "xma_grouped_gemm: MT takes no epilogue");
+        XMA_REQUIRE(a.lda >= a.n && a.ldb >= a.k && a.ldc >= a.k, "xma_grouped_gemm: MT row strides too small");
+        XMA_REQUIRE(a.out_index == nullptr, "xma_grouped_gemm: MT takes no out_index");
+        if (a.n == 0 || a.k == 0) return 0;
+    } else {
+        XMA_REQUIRE(a.epilogue == XMA_EPI_NONE || (a.kind == XMA_GEMM_TN && a.epilogue == XMA_EPI_SWIGLU) ||
+                        (a.kind == XMA_GEMM_NN && a.epilogue == XMA_EPI_SWIGLU_BWD),
+                    "xma_grouped_gemm: epilogue %d not available for kind %d", a.epilogue, a.kind);
+        XMA_REQUIRE(a.lda >= a.k, "xma_grouped_gemm: lda too small");
+        XMA_REQUIRE(a.ldb >= (a.kind == XMA_GEMM_TN ? a.k : a.n), "xma_grouped_gemm: ldb too small");
+        if (a.epilogue == XMA_EPI_SWIGLU) {
+            XMA_REQUIRE(a.n % (2 * pv) == 0, "xma_grouped_gemm: SwiGLU epilogue needs n %% %d == 0", 2 * pv);
+            XMA_REQUIRE(a.ldc >= a.n / 2, "xma_grouped_gemm: ldc too small");
+            XMA_REQUIRE(a.aux == nullptr || a.ld_aux >= a.n, "xma_grouped_gemm: ld_aux too small");
+        } else if (a.epilogue == XMA_EPI_SWIGLU_BWD) {
+            XMA_REQUIRE(a.aux != nullptr && a.ld_aux >= 2 * a.n && a.ldc >= 2 * a.n,
+                        "xma_grouped_gemm: SwiGLU backward epilogue needs aux/ldc of 2n columns");
+            XMA_REQUIRE(a.out_index == nullptr, "xma_grouped_gemm: SwiGLU backward epilogue writes grouped rows");
+        } else {
+            XMA_REQUIRE(a.ldc >= a.n, "xma_grouped_gemm: ldc too small");
+        }
+        if (a.rows == 0 || a.n == 0) return 0;
+        XMA_REQUIRE(a.workspace != nullptr &&
+                        a.workspace_bytes >= xma_grouped_gemm_workspace_bytes(a.num_experts, a.rows),
+                    "xma_grouped_gemm: workspace too small (%lld < %lld)", (long long)a.workspace_bytes,
+                    (long long)xma_grouped_gemm_workspace_bytes(a.num_experts, a.rows));
+    }
+    XMA_REQUIRE(a.a && a.b && a.c, "xma_grouped_gemm: null operand");
+    hipStream_t stream = (hipStream_t)stream_;
+    switch (a.dtype) {
+        case XMA_F32:
+            return dispatch_kind<float>(a, stream);
+        case XMA_F16:
+            return dispatch_kind<f16_t>(a, stream);
+        default:
+            return dispatch_kind<bf16_t>(a, stream);
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,509 @@
+// Routing metadata for the MoE layer on gfx950: expert histogram (continuous_count), exclusive
+// offsets, stable counting-sort permutation, and the router's top-k + softmax (forward and
+// backward).  All integer results are order-independent or explicitly ordered, so they are
+// bit-exact from run to run.
+//
+// Work decomposition of the counting sort: the id stream is cut into contiguous chunks of
+// kChunk ids, one wavefront per chunk.  (1) every wave builds a private histogram of its
+// chunk in LDS and writes it out as a row of `unit_hist[units][E]`; (2) a column-wise
+// exclusive scan over the units plus an exclusive scan over the experts turn the rows into
+// the first output slot of every (unit, expert) pair; (3) every wave walks its chunk again in
+// order, ranks equal ids inside each 64-wide batch with ballots, and writes the permutation.
+#include "common.h"
+
+namespace xma {
+
+constexpr int kChunk = 1024;        // ids per wave-unit of the counting sort
+constexpr int kMaxExperts = 16384;  // same limit as the reference kernel (forward.cu:12)
+
+// ------------------------------------------------------------------------------------------
+// continuous_count
+// ------------------------------------------------------------------------------------------
+__global__ void fill_u32_kernel(uint32_t* p, int64_t n, uint32_t v) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// LDS holds `copies` replicas of the histogram (stride `bins`); lane l uses replica l % copies,
+// which divides the same-address serialisation of LDS atomics when there are few bins.
+template <typename IdT>
+__global__ __launch_bounds__(256) void count_kernel(const IdT* __restrict__ ids, int64_t n, int bins,
+                                                     int copies, int vec_ok, uint32_t* __restrict__ counts) {
+    extern __shared__ uint32_t lds_hist[];
+    const int total = bins * copies;
+    for (int i = threadIdx.x; i < total; i += blockDim.x) lds_hist[i] = 0;
+    __syncthreads();
+
+    uint32_t* mine = lds_hist + (threadIdx.x % copies) * bins;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+    constexpr int kPerVec = 16 / sizeof(IdT);
+
+    if (vec_ok) {
+        const int64_t nvec = n / kPerVec;
+        const uint4* v = reinterpret_cast<const uint4*>(ids);
+        for (int64_t i = tid; i < nvec; i += nthreads) {
+            uint4 q = v[i];
+            IdT e[kPerVec];
+            if constexpr (sizeof(IdT) == 4) {
+                e[0] = (IdT)q.x;
+                e[1] = (IdT)q.y;
+                e[2] = (IdT)q.z;
+                e[3] = (IdT)q.w;
+            } else {
+                e[0] = (IdT)(((uint64_t)q.y << 32) | q.x);
+                e[1] = (IdT)(((uint64_t)q.w << 32) | q.z);
+            }
+#pragma unroll
+            for (int j = 0; j < kPerVec; ++j)
+                if (e[j] >= 0 && e[j] < bins) atomicAdd(&mine[e[j]], 1u);
+        }
+        for (int64_t i = nvec * kPerVec + tid; i < n; i += nthreads) {
+            IdT e = ids[i];
+            if (e >= 0 && e < bins) atomicAdd(&mine[e], 1u);
+        }
+    } else {
+        for (int64_t i = tid; i < n; i += nthreads) {
+            IdT e = ids[i];
+            if (e >= 0 && e < bins) atomicAdd(&mine[e], 1u);
+        }
+    }
+    __syncthreads();
+
+    for (int b = threadIdx.x; b < bins; b += blockDim.x) {
+        uint32_t c = 0;
+        for (int r = 0; r < copies; ++r) c += lds_hist[r * bins + b];
+        if (c) atomicAdd(&counts[b], c);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// stable counting sort
+// ------------------------------------------------------------------------------------------
+template <typename IdT>
+__global__ __launch_bounds__(256) void unit_hist_kernel(const IdT* __restrict__ ids, int64_t n, int E,
+                                                         int waves_per_block, uint32_t* __restrict__ unit_hist) {
+    extern __shared__ uint32_t lds_hist[];
+    const int wave = threadIdx.x / kWaveSize;
+    const int lane = lane_id();
+    uint32_t* mine = lds_hist + wave * E;
+    for (int i = lane; i < E; i += kWaveSize) mine[i] = 0;
+    __syncthreads();
+    const int64_t unit = (int64_t)blockIdx.x * waves_per_block + wave;
+    const int64_t begin = unit * kChunk;
+    if (begin < n) {
+        const int64_t end = begin + kChunk < n ? begin + kChunk : n;
+        for (int64_t i = begin + lane; i < end; i += kWaveSize) {
+            IdT e = ids[i];
+            if (e >= 0 && e < E) atomicAdd(&mine[e], 1u);
+        }
+    }
+    __syncthreads();
+    if (begin < n) {
+        uint32_t* row = unit_hist + unit * E;
+        for (int i = lane; i < E; i += kWaveSize) row[i] = mine[i];
+    }
+}
+
+// One block of 16 waves per 64 experts: lane = expert column, wave = a segment of the units.
+// In place: unit_hist[u][e] becomes the number of ids equal to e in units before u; the column
+// totals go to counts[e].
+__global__ __launch_bounds__(1024) void unit_scan_kernel(uint32_t* __restrict__ unit_hist, int64_t units, int E,
+                                                          uint32_t* __restrict__ counts) {
+    __shared__ uint32_t seg_sum[16][kWaveSize];
+    const int wave = threadIdx.x / kWaveSize;
+    const int lane = lane_id();
+    const int e = blockIdx.x * kWaveSize + lane;
+    const int64_t seg = (units + 15) / 16;
+    const int64_t u0 = wave * seg;
+    const int64_t u1 = u0 + seg < units ? u0 + seg : units;
+    uint32_t s = 0;
+    if (e < E)
+        for (int64_t u = u0; u < u1; ++u) s += unit_hist[u * E + e];
+    seg_sum[wave][lane] = s;
+    __syncthreads();
+    uint32_t base = 0;
+    for (int w = 0; w < wave; ++w) base += seg_sum[w][lane];
+    if (e < E) {
+        for (int64_t u = u0; u < u1; ++u) {
+            uint32_t c = unit_hist[u * E + e];
+            unit_hist[u * E + e] = base;
+            base += c;
+        }
+        if (wave == 15) counts[e] = base;
+    }
+}
+
+// Single block: offsets[0..E] = exclusive scan of counts[0..E).
+__global__ __launch_bounds__(1024) void offsets_kernel(const uint32_t* __restrict__ counts, int E,
+                                                        int32_t* __restrict__ offsets) {
+    __shared__ uint32_t part[1024];
+    const int per = (E + 1023) / 1024;  // <= 16
+    const int b = threadIdx.x * per;
+    uint32_t s = 0;
+    for (int i = 0; i < per; ++i)
+        if (b + i < E) s += counts[b + i];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    // Hillis-Steele inclusive scan over the 1024 partial sums
+    for (int d = 1; d < 1024; d <<= 1) {
+        uint32_t v = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+        __syncthreads();
+        part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    uint32_t run = part[threadIdx.x] - s;
+    for (int i = 0; i < per; ++i) {
+        if (b + i < E) {
+            offsets[b + i] = (int32_t)run;
+            run += counts[b + i];
+        }
+    }
+    if (threadIdx.x == 1023) offsets[E] = (int32_t)part[1023];
+}
+
+template <typename IdT, typename OutT>
+__global__ __launch_bounds__(256) void place_kernel(const IdT* __restrict__ ids, int64_t n, int E, int nbits,
+                                                     int waves_per_block, const uint32_t* __restrict__ unit_prefix,
+                                                     const int32_t* __restrict__ offsets, OutT* __restrict__ sorted_ids,
+                                                     OutT* __restrict__ perm) {
+    extern __shared__ uint32_t lds_hist[];
+    const int wave = threadIdx.x / kWaveSize;
+    const int lane = lane_id();
+    uint32_t* next = lds_hist + wave * E;  // next free output slot per expert, private to this wave
+    const int64_t unit = (int64_t)blockIdx.x * waves_per_block + wave;
+    const int64_t begin = unit * kChunk;
+    if (begin >= n) return;  // no block-wide barrier below, so whole waves may leave
+    const uint32_t* row = unit_prefix + unit * E;
+    for (int i = lane; i < E; i += kWaveSize) next[i] = row[i] + (uint32_t)offsets[i];
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+
+    const int64_t end = begin + kChunk < n ? begin + kChunk : n;
+    const uint64_t lt_mask = ((uint64_t)1 << lane) - 1;
+    for (int64_t i0 = begin; i0 < end; i0 += kWaveSize) {
+        const int64_t i = i0 + lane;
+        const bool live = i < end;
+        int64_t e64 = live ? (int64_t)ids[i] : -1;
+        const bool ok = live && e64 >= 0 && e64 < E;
+        const uint32_t e = ok ? (uint32_t)e64 : 0u;
+        // lanes holding the same expert id as this lane
+        uint64_t peers = __ballot(ok);
+        for (int b = 0; b < nbits; ++b) {
+            const bool bit = (e >> b) & 1u;
+            const uint64_t bal = __ballot(ok && bit);
+            peers &= bit ? bal : ~bal;
+        }
+        uint32_t base = 0;
+        const int leader = ok ? (int)__ffsll((unsigned long long)peers) - 1 : lane;
+        if (ok && leader == lane) {
+            base = next[e];
+            next[e] = base + (uint32_t)__popcll(peers);
+        }
+        base = __shfl(base, leader, kWaveSize);
+        if (ok) {
+            const uint32_t pos = base + (uint32_t)__popcll(peers & lt_mask);
+            perm[pos] = (OutT)i;
+            sorted_ids[pos] = (OutT)e;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// router top-k + softmax
+// ------------------------------------------------------------------------------------------
+// Monotone map float -> uint32 (larger float => larger key); NaN above +inf; -0 == +0.
+__device__ __forceinline__ uint32_t order_key(float v) {
+    if (v != v) return 0xffffffffu;
+    if (v == 0.0f) v = 0.0f;
+    uint32_t u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_to_float(uint32_t key) {
+    return __uint_as_float((key & 0x80000000u) ? (key ^ 0x80000000u) : ~key);
+}
+
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+#pragma unroll
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) {
+        uint32_t lo = __shfl_xor((uint32_t)v, off, kWaveSize);
+        uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, kWaveSize);
+        uint64_t o = ((uint64_t)hi << 32) | lo;
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
+// One wave per token; lane l owns experts l, l+64, ...  (EPL per lane, E <= 64*EPL).
+// key = (order_key(value) << 32) | (0xffffffff - expert): the maximum picks the largest value
+// and, among equals, the lowest expert index.
+template <typename T, int EPL, typename IdxT>
+__global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__ logits, int64_t Tn, int E, int k,
+                                                            int64_t ld, T* __restrict__ weights,
+                                                            IdxT* __restrict__ idx) {
+    const int lane = lane_id();
+    const int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize;
+    if (t >= Tn) return;
+    const T* row = logits + t * ld;
+    uint64_t keys[EPL];
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+        const int e = lane + j * kWaveSize;
+        keys[j] = e < E ? (((uint64_t)order_key(Elem<T>::load(row + e)) << 32) | (uint32_t)(0xffffffffu - (uint32_t)e))
+                        : 0ull;
+    }
+    float my_val = 0.0f;
+    uint32_t my_idx = 0;
+    float vmax = 0.0f;
+    for (int s = 0; s < k; ++s) {
+        uint64_t best = 0;
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) best = keys[j] > best ? keys[j] : best;
+        best = wave_max_u64(best);
+#pragma unroll
+        for (int j = 0; j < EPL; ++j)
+            if (keys[j] == best) keys[j] = 0ull;
+        const float v = key_to_float((uint32_t)(best >> 32));
+        if (s == 0) vmax = v;
+        if (lane == s) {
+            my_val = v;
+            my_idx = 0xffffffffu - (uint32_t)best;
+        }
+    }
+    const float ex = lane < k ? expf(my_val - vmax) : 0.0f;
+    const float denom = wave_sum(ex);
+    if (lane < k) {
+        Elem<T>::store(weights + t * k + lane, ex / denom);
+        idx[t * k + lane] = (IdxT)my_idx;
+    }
+}
+
+// Any E <= 16384: one wave per block, ordered keys of the row staged in LDS.
+template <typename T, typename IdxT>
+__global__ __launch_bounds__(64) void topk_softmax_lds_kernel(const T* __restrict__ logits, int64_t Tn, int E, int k,
+                                                               int64_t ld, T* __restrict__ weights,
+                                                               IdxT* __restrict__ idx) {
+    extern __shared__ uint32_t lds_keys[];
+    const int lane = lane_id();
+    const int64_t t = blockIdx.x;
+    const T* row = logits + t * ld;
+    for (int e = lane; e < E; e += kWaveSize) lds_keys[e] = order_key(Elem<T>::load(row + e));
+    __syncthreads();
+    float my_val = 0.0f, vmax = 0.0f;
+    uint32_t my_idx = 0;
+    for (int s = 0; s < k; ++s) {
+        uint64_t best = 0;
+        for (int e = lane; e < E; e += kWaveSize) {
+            const uint32_t kk = lds_keys[e];
+            // order_key never returns 0 (its minimum, for -inf, is 0x007fffff): 0 marks a taken slot
+            uint64_t key = ((uint64_t)kk << 32) | (uint32_t)(0xffffffffu - (uint32_t)e);
+            if (kk == 0u) key = 0ull;
+            best = key > best ? key : best;
+        }
+        best = wave_max_u64(best);
+        const uint32_t win = 0xffffffffu - (uint32_t)best;
+        if (lane == 0 && best != 0ull) lds_keys[win] = 0u;
+        __syncthreads();
+        const float v = key_to_float((uint32_t)(best >> 32));
+        if (s == 0) vmax = v;
+        if (lane == s) {
+            my_val = v;
+            my_idx = win;
+        }
+    }
+    const float ex = lane < k ? expf(my_val - vmax) : 0.0f;
+    const float denom = wave_sum(ex);
+    if (lane < k) {
+        Elem<T>::store(weights + t * k + lane, ex / denom);
+        idx[t * k + lane] = (IdxT)my_idx;
+    }
+}
+
+// d_logits[t, :] = 0, then d_logits[t, idx[t, j]] = w_j * (dw_j - sum_i w_i dw_i) with
+// w = softmax(logits[t, idx[t, :]]) recomputed in fp32.  One wave per token.
+template <typename T, typename IdxT>
+__global__ __launch_bounds__(256) void topk_softmax_bwd_kernel(const T* __restrict__ logits, int64_t ld_logits,
+                                                                const T* __restrict__ d_weights,
+                                                                const IdxT* __restrict__ idx, int64_t Tn, int E, int k,
+                                                                T* __restrict__ d_logits, int64_t ld) {
+    const int lane = lane_id();
+    const int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize;
+    if (t >= Tn) return;
+    T* out = d_logits + t * ld;
+    for (int e = lane; e < E; e += kWaveSize) Elem<T>::store(out + e, 0.0f);
+    int64_t e_sel = 0;
+    float v = -INFINITY, dw = 0.0f;
+    if (lane < k) {
+        e_sel = (int64_t)idx[t * k + lane];
+        v = Elem<T>::load(logits + t * ld_logits + e_sel);
+        dw = Elem<T>::load(d_weights + t * k + lane);
+    }
+    float vmax = v;
+#pragma unroll
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, off, kWaveSize));
+    const float ex = lane < k ? expf(v - vmax) : 0.0f;
+    const float w = ex / wave_sum(ex);
+    const float dot = wave_sum(w * dw);
+    // the zero fill above and this store touch the same addresses from different lanes
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (lane < k) Elem<T>::store(out + e_sel, w * (dw - dot));
+}
+
+static int ceil_log2(int v) {
+    int b = 0;
+    while ((1 << b) < v) ++b;
+    return b;
+}
+
+static int sort_waves_per_block(int E) {
+    int w = 16384 / E;  // 64 KiB of LDS histograms per block
+    if (w > 4) w = 4;
+    if (w < 1) w = 1;
+    return w;
+}
+
+}  // namespace xma
+
+using namespace xma;
+
+extern "C" {
+
+int xma_continuous_count(const void* ids, int ids_is_i64, int64_t n, int32_t bins, uint32_t* counts,
+                         void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    XMA_REQUIRE(bins >= 1 && bins <= kMaxExperts, "xma_continuous_count: bins=%d outside [1, %d]", bins, kMaxExperts);
+    XMA_REQUIRE(n >= 0 && n < ((int64_t)1 << 32), "xma_continuous_count: n=%lld does not fit uint32", (long long)n);
+    XMA_REQUIRE(counts != nullptr && (ids != nullptr || n == 0), "xma_continuous_count: null pointer");
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((bins + 255) / 256), dim3(256), 0, stream, counts, (int64_t)bins, 0u);
+    if (n > 0) {
+        int copies = 2048 / bins;
+        if (copies > 32) copies = 32;
+        if (copies < 1) copies = 1;
+        const int per_block = 256 * 16;
+        int64_t blocks = ceil_div(n, per_block);
+        if (blocks > 2048) blocks = 2048;
+        const size_t lds = (size_t)bins * copies * sizeof(uint32_t);
+        const int vec_ok = aligned16(ids) ? 1 : 0;
+        if (ids_is_i64)
+            hipLaunchKernelGGL(count_kernel<int64_t>, dim3((unsigned)blocks), dim3(256), lds, stream,
+                               (const int64_t*)ids, n, (int)bins, copies, vec_ok, counts);
+        else
+            hipLaunchKernelGGL(count_kernel<int32_t>, dim3((unsigned)blocks), dim3(256), lds, stream,
+                               (const int32_t*)ids, n, (int)bins, copies, vec_ok, counts);
+    }
+    return check_launch("xma_continuous_count");
+}
+
+int64_t xma_route_workspace_bytes(int64_t n, int32_t num_experts) {
+    if (n < 0 || num_experts < 1) return -1;
+    const int64_t units = ceil_div(n > 0 ? n : 1, kChunk);
+    return units * (int64_t)num_experts * (int64_t)sizeof(uint32_t);
+}
+
+int xma_route_build(const void* ids, int ids_is_i64, int64_t n, int32_t E, uint32_t* counts, int32_t* offsets,
+                    void* sorted_ids, void* perm, int out_is_i64, void* workspace, int64_t workspace_bytes,
+                    void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    XMA_REQUIRE(E >= 1 && E <= kMaxExperts, "xma_route_build: num_experts=%d outside [1, %d]", E, kMaxExperts);
+    XMA_REQUIRE(n >= 0 && n < ((int64_t)1 << 31), "xma_route_build: n=%lld does not fit int32", (long long)n);
+    XMA_REQUIRE(counts && offsets, "xma_route_build: counts/offsets must not be null");
+    XMA_REQUIRE(n == 0 || (ids && sorted_ids && perm && workspace), "xma_route_build: null pointer");
+    XMA_REQUIRE(workspace_bytes >= xma_route_workspace_bytes(n, E), "xma_route_build: workspace too small (%lld < %lld)",
+                (long long)workspace_bytes, (long long)xma_route_workspace_bytes(n, E));
+    if (n == 0) {
+        hipLaunchKernelGGL(fill_u32_kernel, dim3((E + 255) / 256), dim3(256), 0, stream, counts, (int64_t)E, 0u);
+        hipLaunchKernelGGL(fill_u32_kernel, dim3((E + 1 + 255) / 256), dim3(256), 0, stream, (uint32_t*)offsets,
+                           (int64_t)E + 1, 0u);
+        return check_launch("xma_route_build");
+    }
+    const int64_t units = ceil_div(n, kChunk);
+    const int wpb = sort_waves_per_block(E);
+    const unsigned blocks = (unsigned)ceil_div(units, wpb);
+    const size_t lds = (size_t)wpb * E * sizeof(uint32_t);
+    uint32_t* unit_hist = (uint32_t*)workspace;
+    if (ids_is_i64)
+        hipLaunchKernelGGL(unit_hist_kernel<int64_t>, dim3(blocks), dim3(wpb * kWaveSize), lds, stream,
+                           (const int64_t*)ids, n, (int)E, wpb, unit_hist);
+    else
+        hipLaunchKernelGGL(unit_hist_kernel<int32_t>, dim3(blocks), dim3(wpb * kWaveSize), lds, stream,
+                           (const int32_t*)ids, n, (int)E, wpb, unit_hist);
+    hipLaunchKernelGGL(unit_scan_kernel, dim3((E + kWaveSize - 1) / kWaveSize), dim3(1024), 0, stream, unit_hist, units,
+                       (int)E, counts);
+    hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, stream, (const uint32_t*)counts, (int)E, offsets);
+    const int nbits = ceil_log2(E);
+#define XMA_PLACE(IdT, OutT)                                                                                       \
+    hipLaunchKernelGGL((place_kernel<IdT, OutT>), dim3(blocks), dim3(wpb * kWaveSize), lds, stream, (const IdT*)ids, \
+                       n, (int)E, nbits, wpb, (const uint32_t*)unit_hist, (const int32_t*)offsets,                 \
+                       (OutT*)sorted_ids, (OutT*)perm)
+    if (ids_is_i64) {
+        if (out_is_i64)
+            XMA_PLACE(int64_t, int64_t);
+        else
+            XMA_PLACE(int64_t, int32_t);
+    } else {
+        if (out_is_i64)
+            XMA_PLACE(int32_t, int64_t);
+        else
+            XMA_PLACE(int32_t, int32_t);
+    }
+#undef XMA_PLACE
+    return check_launch("xma_route_build");
+}
+
+int xma_topk_softmax(const void* logits, int dtype, int64_t T, int32_t E, int32_t k, int64_t ld, void* weights,
+                     void* idx, int idx_is_i64, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    XMA_REQUIRE(valid_dtype(dtype), "xma_topk_softmax: bad dtype %d", dtype);
+    XMA_REQUIRE(E >= 1 && E <= kMaxExperts, "xma_topk_softmax: E=%d outside [1, %d]", E, kMaxExperts);
+    XMA_REQUIRE(k >= 1 && k <= E && k <= kWaveSize, "xma_topk_softmax: k=%d must satisfy 1 <= k <= min(E=%d, 64)", k, E);
+    XMA_REQUIRE(T >= 0 && ld >= E, "xma_topk_softmax: bad T=%lld or row stride %lld", (long long)T, (long long)ld);
+    if (T == 0) return 0;
+    XMA_REQUIRE(logits && weights && idx, "xma_topk_softmax: null pointer");
+    const int wpb = 4;
+    const unsigned blocks = (unsigned)ceil_div(T, wpb);
+#define XMA_TOPK(T_, EPL, IdxT)                                                                                    \
+    hipLaunchKernelGGL((topk_softmax_kernel<T_, EPL, IdxT>), dim3(blocks), dim3(wpb * kWaveSize), 0, stream,        \
+                       (const T_*)logits, T, (int)E, (int)k, ld, (T_*)weights, (IdxT*)idx)
+#define XMA_TOPK_E(T_, IdxT)                                                                                       \
+    if (E <= 64)                                                                                                   \
+        XMA_TOPK(T_, 1, IdxT);                                                                                     \
+    else if (E <= 128)                                                                                             \
+        XMA_TOPK(T_, 2, IdxT);                                                                                     \
+    else if (E <= 256)                                                                                             \
+        XMA_TOPK(T_, 4, IdxT);                                                                                     \
+    else if (E <= 512)                                                                                             \
+        XMA_TOPK(T_, 8, IdxT);                                                                                     \
+    else                                                                                                           \
+        hipLaunchKernelGGL((topk_softmax_lds_kernel<T_, IdxT>), dim3((unsigned)T), dim3(kWaveSize),                \
+                           (size_t)E * sizeof(uint32_t), stream, (const T_*)logits, T, (int)E, (int)k, ld,         \
+                           (T_*)weights, (IdxT*)idx)
+    XMA_DISPATCH_DTYPE(dtype, T_, if (idx_is_i64) { XMA_TOPK_E(T_, int64_t); } else { XMA_TOPK_E(T_, int32_t); })
+#undef XMA_TOPK_E
+#undef XMA_TOPK
+    return check_launch("xma_topk_softmax");
+}
+
+int xma_topk_softmax_bwd(const void* logits, int64_t ld_logits, const void* d_weights, const void* idx,
+                         int idx_is_i64, int dtype, int64_t T, int32_t E, int32_t k, void* d_logits, int64_t ld,
+                         void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    XMA_REQUIRE(valid_dtype(dtype), "xma_topk_softmax_bwd: bad dtype %d", dtype);
+    XMA_REQUIRE(E >= 1 && k >= 1 && k <= E && k <= kWaveSize, "xma_topk_softmax_bwd: bad E=%d / k=%d", E, k);
+    XMA_REQUIRE(T >= 0 && ld >= E && ld_logits >= E, "xma_topk_softmax_bwd: bad T or row stride");
+    if (T == 0) return 0;
+    XMA_REQUIRE(logits && d_weights && idx && d_logits, "xma_topk_softmax_bwd: null pointer");
+    const int wpb = 4;
+    const unsigned blocks = (unsigned)ceil_div(T, wpb);
+    XMA_DISPATCH_DTYPE(
+        dtype, T_,
+        if (idx_is_i64) hipLaunchKernelGGL((topk_softmax_bwd_kernel<T_, int64_t>), dim3(blocks), dim3(wpb * kWaveSize),
+                                           0, stream, (const T_*)logits, ld_logits, (const T_*)d_weights,
+                                           (const int64_t*)idx, T, (int)E, (int)k, (T_*)d_logits, ld);
+        else hipLaunchKernelGGL((topk_softmax_bwd_kernel<T_, int32_t>), dim3(blocks), dim3(wpb * kWaveSize), 0, stream,
+                                (const T_*)logits, ld_logits, (const T_*)d_weights, (const int32_t*)idx, T, (int)E,
+                                (int)k, (T_*)d_logits, ld))
+    return check_launch("xma_topk_softmax_bwd");
+}
+
+}  // extern "C"

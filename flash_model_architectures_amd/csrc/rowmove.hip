@@ -1,0 +1,276 @@
+// HBM-bound row kernels of the MoE layer on gfx950: token gather (permute) with optional
+// per-row coefficient, row scatter (unpermute), top-k weighted combine / fold, and the gate
+// gradient.  Rows are moved as 16-byte vectors; a block walks kRowsPerIter rows at a time so
+// that several independent loads are in flight per lane before the first store.
+#include "common.h"
+
+namespace xma {
+
+constexpr int kRowsPerIter = 4;
+
+enum RowMode { kGather = 0, kScatter = 1 };
+
+// 16-byte path: cols is a multiple of Elem<T>::kPerVec, strides keep rows 16-byte aligned.
+template <typename T, int MODE, bool COEFF>
+__global__ __launch_bounds__(256) void move_rows_vec_kernel(const T* __restrict__ src, int64_t ld_src,
+                                                             T* __restrict__ dst, int64_t ld_dst,
+                                                             const void* __restrict__ index, int idx_is_i64,
+                                                             int64_t rows, int chunks, int fan_out,
+                                                             const T* __restrict__ coeff) {
+    constexpr int PV = Elem<T>::kPerVec;
+    for (int64_t r0 = (int64_t)blockIdx.x * kRowsPerIter; r0 < rows; r0 += (int64_t)gridDim.x * kRowsPerIter) {
+        int64_t srow[kRowsPerIter], drow[kRowsPerIter];
+        float scale[kRowsPerIter];
+#pragma unroll
+        for (int j = 0; j < kRowsPerIter; ++j) {
+            const int64_t p = r0 + j < rows ? r0 + j : rows - 1;
+            const int64_t ix = index ? load_index(index, idx_is_i64, p) : p;
+            srow[j] = MODE == kGather ? ix / fan_out : p;
+            drow[j] = MODE == kGather ? p : ix;
+            scale[j] = 1.0f;
+            if constexpr (COEFF) scale[j] = Elem<T>::load(coeff + ix);
+        }
+        for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
+            uint4 v[kRowsPerIter];
+#pragma unroll
+            for (int j = 0; j < kRowsPerIter; ++j)
+                v[j] = *reinterpret_cast<const uint4*>(src + srow[j] * ld_src + (int64_t)c * PV);
+#pragma unroll
+            for (int j = 0; j < kRowsPerIter; ++j) {
+                if constexpr (COEFF) {
+                    float f[PV];
+                    Elem<T>::unpack(v[j], f);
+#pragma unroll
+                    for (int q = 0; q < PV; ++q) f[q] *= scale[j];
+                    v[j] = Elem<T>::pack(f);
+                }
+                if (r0 + j < rows) *reinterpret_cast<uint4*>(dst + drow[j] * ld_dst + (int64_t)c * PV) = v[j];
+            }
+        }
+    }
+}
+
+// element-wise path for odd widths or unaligned views
+template <typename T, int MODE, bool COEFF>
+__global__ __launch_bounds__(256) void move_rows_scalar_kernel(const T* __restrict__ src, int64_t ld_src,
+                                                                T* __restrict__ dst, int64_t ld_dst,
+                                                                const void* __restrict__ index, int idx_is_i64,
+                                                                int64_t rows, int64_t cols, int fan_out,
+                                                                const T* __restrict__ coeff) {
+    for (int64_t p = blockIdx.x; p < rows; p += gridDim.x) {
+        const int64_t ix = index ? load_index(index, idx_is_i64, p) : p;
+        const int64_t srow = MODE == kGather ? ix / fan_out : p;
+        const int64_t drow = MODE == kGather ? p : ix;
+        float scale = 1.0f;
+        if constexpr (COEFF) scale = Elem<T>::load(coeff + ix);
+        for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+            if constexpr (COEFF)
+                Elem<T>::store(dst + drow * ld_dst + c, Elem<T>::load(src + srow * ld_src + c) * scale);
+            else
+                dst[drow * ld_dst + c] = src[srow * ld_src + c];
+        }
+    }
+}
+
+// y[t, :] = sum_j gates[t, j] * y_exp[t*k + j, :]   (GATED) or the plain sum over j.
+template <typename T, bool GATED, bool VEC>
+__global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y_exp, int64_t ld_exp,
+                                                       const T* __restrict__ gates, T* __restrict__ y, int64_t ld_y,
+                                                       int64_t Tn, int k, int64_t cols) {
+    constexpr int PV = VEC ? Elem<T>::kPerVec : 1;
+    const int64_t chunks = cols / PV;
+    for (int64_t t = blockIdx.x; t < Tn; t += gridDim.x) {
+        const T* base = y_exp + t * k * ld_exp;
+        for (int64_t c = threadIdx.x; c < chunks; c += blockDim.x) {
+            float acc[PV];
+#pragma unroll
+            for (int q = 0; q < PV; ++q) acc[q] = 0.0f;
+            int j = 0;
+            if constexpr (VEC) {
+                for (; j + 2 <= k; j += 2) {
+                    const uint4 v0 = *reinterpret_cast<const uint4*>(base + (int64_t)j * ld_exp + c * PV);
+                    const uint4 v1 = *reinterpret_cast<const uint4*>(base + (int64_t)(j + 1) * ld_exp + c * PV);
+                    float f0[PV], f1[PV];
+                    Elem<T>::unpack(v0, f0);
+                    Elem<T>::unpack(v1, f1);
+                    const float g0 = GATED ? Elem<T>::load(gates + t * k + j) : 1.0f;
+                    const float g1 = GATED ? Elem<T>::load(gates + t * k + j + 1) : 1.0f;
+#pragma unroll
+                    for (int q = 0; q < PV; ++q) acc[q] = fmaf(g0, f0[q], acc[q]);
+#pragma unroll
+                    for (int q = 0; q < PV; ++q) acc[q] = fmaf(g1, f1[q], acc[q]);
+                }
+            }
+            for (; j < k; ++j) {
+                const float g = GATED ? Elem<T>::load(gates + t * k + j) : 1.0f;
+                if constexpr (VEC) {
+                    const uint4 v = *reinterpret_cast<const uint4*>(base + (int64_t)j * ld_exp + c * PV);
+                    float f[PV];
+                    Elem<T>::unpack(v, f);
+#pragma unroll
+                    for (int q = 0; q < PV; ++q) acc[q] = fmaf(g, f[q], acc[q]);
+                } else {
+                    acc[0] = fmaf(g, Elem<T>::load(base + (int64_t)j * ld_exp + c), acc[0]);
+                }
+            }
+            if constexpr (VEC)
+                *reinterpret_cast<uint4*>(y + t * ld_y + c * PV) = Elem<T>::pack(acc);
+            else
+                Elem<T>::store(y + t * ld_y + c, acc[0]);
+        }
+    }
+}
+
+// d_gates[t, j] = <y_exp[t*k + j, :], dy[t, :]>; block per token, wave per slot j.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void gate_grad_kernel(const T* __restrict__ y_exp, int64_t ld_exp,
+                                                         const T* __restrict__ dy, int64_t ld_dy,
+                                                         T* __restrict__ d_gates, int64_t Tn, int k, int64_t cols) {
+    constexpr int PV = VEC ? Elem<T>::kPerVec : 1;
+    const int64_t chunks = cols / PV;
+    const int wave = threadIdx.x / kWaveSize;
+    const int nwaves = blockDim.x / kWaveSize;
+    const int lane = lane_id();
+    for (int64_t t = blockIdx.x; t < Tn; t += gridDim.x) {
+        for (int j = wave; j < k; j += nwaves) {
+            const T* row = y_exp + (t * k + j) * ld_exp;
+            const T* g = dy + t * ld_dy;
+            float acc = 0.0f;
+            for (int64_t c = lane; c < chunks; c += kWaveSize) {
+                if constexpr (VEC) {
+                    float a[PV], b[PV];
+                    Elem<T>::unpack(*reinterpret_cast<const uint4*>(row + c * PV), a);
+                    Elem<T>::unpack(*reinterpret_cast<const uint4*>(g + c * PV), b);
+#pragma unroll
+                    for (int q = 0; q < PV; ++q) acc = fmaf(a[q], b[q], acc);
+                } else {
+                    acc = fmaf(Elem<T>::load(row + c), Elem<T>::load(g + c), acc);
+                }
+            }
+            acc = wave_sum(acc);
+            if (lane == 0) Elem<T>::store(d_gates + t * k + j, acc);
+        }
+    }
+}
+
+static unsigned row_grid(int64_t work_items) {
+    const int64_t cap = 256 * 16;  // 256 CUs, up to 16 resident blocks of 256 threads each
+    int64_t g = work_items < cap ? work_items : cap;
+    return (unsigned)(g < 1 ? 1 : g);
+}
+
+static unsigned row_block(int64_t chunks) {
+    int64_t b = ((chunks + kWaveSize - 1) / kWaveSize) * kWaveSize;
+    if (b > 256) b = 256;
+    if (b < kWaveSize) b = kWaveSize;
+    return (unsigned)b;
+}
+
+template <typename T>
+static bool vec_ok(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t cols) {
+    constexpr int PV = Elem<T>::kPerVec;
+    return aligned16(a) && aligned16(b) && lda % PV == 0 && ldb % PV == 0 && cols % PV == 0;
+}
+
+template <typename T, int MODE>
+static void launch_move(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, const void* index,
+                        int idx_is_i64, int64_t rows, int64_t cols, int fan_out, const void* coeff,
+                        hipStream_t stream) {
+    constexpr int PV = Elem<T>::kPerVec;
+    if (vec_ok<T>(src, ld_src, dst, ld_dst, cols)) {
+        const int chunks = (int)(cols / PV);
+        const dim3 grid(row_grid(ceil_div(rows, kRowsPerIter))), block(row_block(chunks));
+        if (coeff)
+            hipLaunchKernelGGL((move_rows_vec_kernel<T, MODE, true>), grid, block, 0, stream, (const T*)src, ld_src,
+                               (T*)dst, ld_dst, index, idx_is_i64, rows, chunks, fan_out, (const T*)coeff);
+        else
+            hipLaunchKernelGGL((move_rows_vec_kernel<T, MODE, false>), grid, block, 0, stream, (const T*)src, ld_src,
+                               (T*)dst, ld_dst, index, idx_is_i64, rows, chunks, fan_out, (const T*)nullptr);
+    } else {
+        const dim3 grid(row_grid(rows)), block(row_block(cols));
+        if (coeff)
+            hipLaunchKernelGGL((move_rows_scalar_kernel<T, MODE, true>), grid, block, 0, stream, (const T*)src, ld_src,
+                               (T*)dst, ld_dst, index, idx_is_i64, rows, cols, fan_out, (const T*)coeff);
+        else
+            hipLaunchKernelGGL((move_rows_scalar_kernel<T, MODE, false>), grid, block, 0, stream, (const T*)src,
+                               ld_src, (T*)dst, ld_dst, index, idx_is_i64, rows, cols, fan_out, (const T*)nullptr);
+    }
+}
+
+}  // namespace xma
+
+using namespace xma;
+
+extern "C" {
+
+int xma_gather_rows(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, const void* index, int idx_is_i64,
+                    int64_t rows, int64_t cols, int dtype, int32_t fan_out, const void* coeff, void* stream_) {
+    XMA_REQUIRE(valid_dtype(dtype), "xma_gather_rows: bad dtype %d", dtype);
+    XMA_REQUIRE(rows >= 0 && cols >= 0 && ld_src >= cols && ld_dst >= cols, "xma_gather_rows: bad shape");
+    XMA_REQUIRE(fan_out >= 1, "xma_gather_rows: fan_out=%d must be >= 1", fan_out);
+    XMA_REQUIRE(coeff == nullptr || index != nullptr, "xma_gather_rows: coeff needs an index");
+    if (rows == 0 || cols == 0) return 0;
+    XMA_REQUIRE(src && dst, "xma_gather_rows: null pointer");
+    XMA_DISPATCH_DTYPE(dtype, T, (launch_move<T, kGather>(src, ld_src, dst, ld_dst, index, idx_is_i64, rows, cols,
+                                                          fan_out, coeff, (hipStream_t)stream_)))
+    return check_launch("xma_gather_rows");
+}
+
+int xma_scatter_rows(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, const void* index, int idx_is_i64,
+                     int64_t rows, int64_t cols, int dtype, void* stream_) {
+    XMA_REQUIRE(valid_dtype(dtype), "xma_scatter_rows: bad dtype %d", dtype);
+    XMA_REQUIRE(rows >= 0 && cols >= 0 && ld_src >= cols && ld_dst >= cols, "xma_scatter_rows: bad shape");
+    if (rows == 0 || cols == 0) return 0;
+    XMA_REQUIRE(src && dst, "xma_scatter_rows: null pointer");
+    XMA_DISPATCH_DTYPE(dtype, T, (launch_move<T, kScatter>(src, ld_src, dst, ld_dst, index, idx_is_i64, rows, cols, 1,
+                                                           nullptr, (hipStream_t)stream_)))
+    return check_launch("xma_scatter_rows");
+}
+
+int xma_combine_topk(const void* y_exp, int64_t ld_exp, const void* gates, void* y, int64_t ld_y, int64_t T,
+                     int32_t k, int64_t cols, int dtype, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    XMA_REQUIRE(valid_dtype(dtype), "xma_combine_topk: bad dtype %d", dtype);
+    XMA_REQUIRE(T >= 0 && k >= 1 && cols >= 0 && ld_exp >= cols && ld_y >= cols, "xma_combine_topk: bad shape");
+    if (T == 0 || cols == 0) return 0;
+    XMA_REQUIRE(y_exp && y, "xma_combine_topk: null pointer");
+#define XMA_COMBINE(G, V)                                                                           \
+    hipLaunchKernelGGL((combine_kernel<T_, G, V>), grid, block, 0, stream, (const T_*)y_exp, ld_exp, \
+                       (const T_*)gates, (T_*)y, ld_y, T, (int)k, cols)
+    XMA_DISPATCH_DTYPE(
+        dtype, T_, const bool vec = vec_ok<T_>(y_exp, ld_exp, y, ld_y, cols);
+        const int64_t chunks = vec ? cols / Elem<T_>::kPerVec : cols;
+        const dim3 grid(row_grid(T)), block(row_block(chunks));
+        if (gates) {
+            if (vec)
+                XMA_COMBINE(true, true);
+            else
+                XMA_COMBINE(true, false);
+        } else {
+            if (vec)
+                XMA_COMBINE(false, true);
+            else
+                XMA_COMBINE(false, false);
+        })
+#undef XMA_COMBINE
+    return check_launch("xma_combine_topk");
+}
+
+int xma_gate_grad(const void* y_exp, int64_t ld_exp, const void* dy, int64_t ld_dy, void* d_gates, int64_t T,
+                  int32_t k, int64_t cols, int dtype, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    XMA_REQUIRE(valid_dtype(dtype), "xma_gate_grad: bad dtype %d", dtype);
+    XMA_REQUIRE(T >= 0 && k >= 1 && cols >= 0 && ld_exp >= cols && ld_dy >= cols, "xma_gate_grad: bad shape");
+    if (T == 0) return 0;
+    XMA_REQUIRE(y_exp && dy && d_gates, "xma_gate_grad: null pointer");
+    XMA_DISPATCH_DTYPE(
+        dtype, T_, const bool vec = vec_ok<T_>(y_exp, ld_exp, dy, ld_dy, cols);
+        const dim3 grid(row_grid(T)), block(256);
+        if (vec) hipLaunchKernelGGL((gate_grad_kernel<T_, true>), grid, block, 0, stream, (const T_*)y_exp, ld_exp,
+                                    (const T_*)dy, ld_dy, (T_*)d_gates, T, (int)k, cols);
+        else hipLaunchKernelGGL((gate_grad_kernel<T_, false>), grid, block, 0, stream, (const T_*)y_exp, ld_exp,
+                                (const T_*)dy, ld_dy, (T_*)d_gates, T, (int)k, cols))
+    return check_launch("xma_gate_grad");
+}
+
+}  // extern "C"

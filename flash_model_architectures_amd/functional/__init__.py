@@ -1,0 +1,4 @@
+from .continuous_count import continuous_count
+from .routing import route_tokens, topk_softmax
+from .swiglu import swiglu
+from .swiglu_packed import swiglu_packed

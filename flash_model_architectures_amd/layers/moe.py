@@ -1,0 +1,416 @@
+"""Mixture-of-Experts layer over the gfx950 kernels (public surface of xma/layers/moe/__init__.py).
+
+`MoE.forward` = gate linear -> top-k + softmax -> stable counting sort of the (token, slot) pairs
+-> grouped up-projection -> activation -> grouped down-projection scattered back and combined with
+the routing weights.  Two expert pipelines exist:
+
+* `_SwigluExperts`: when the activation is this package's `swiglu_packed`, SwiGLU is fused into the
+  up-projection's epilogue and its backward into the down-projection's input-gradient epilogue.
+* `scattered_experts` (+ any activation callable): the general pipeline with the same call
+  structure as the reference's `_ScatteredExperts`
+  (xma/layers/moe/triton_implementation/__init__.py:14-185).
+"""
+
+from __future__ import annotations
+
+from typing import Callable
+
+import torch
+import torch.nn as nn
+
+from ..accelerator import KernelBackend, resolve_backend
+from ..functional.routing import route_tokens, topk_softmax
+from ..functional.swiglu_packed import swiglu_packed
+from ..ops import (
+    combine_topk,
+    down_projection_dgrad_swiglu,
+    gate_grad,
+    group,
+    group_bwd_W,
+    scatter2scatter,
+    up_projection_swiglu,
+)
+from ..utils import XMAModule
+
+
+class _ScatteredExperts(torch.autograd.Function):
+    """y = experts(x) for one projection; `expert_weights` is the logical [E, in, out] view."""
+
+    @staticmethod
+    def forward(
+        ctx,
+        x,
+        expert_weights,
+        k,
+        sorted_expert_idxs,
+        sorted_scattered_idxs,
+        expert_offsets,
+        gates,
+        grouped_in,
+        grouped_out,
+    ):
+        M = sorted_expert_idxs.size(0)
+        expanded = torch.empty(M, expert_weights.size(-1), device=x.device, dtype=x.dtype)
+        scatter2scatter(
+            X=x,
+            W=expert_weights,
+            sorted_expert_idxs=sorted_expert_idxs,
+            sorted_scattered_idxs=sorted_scattered_idxs,
+            expert_offsets=expert_offsets,
+            out=expanded,
+            FAN_OUT=k,
+            x_grouped=grouped_in,
+            y_grouped=grouped_out,
+        )
+        if gates is None:
+            output, saved_expanded = expanded, None
+        else:
+            # rows t*top_k .. t*top_k + top_k - 1 of `expanded` belong to token t
+            output = torch.empty(gates.size(0), expanded.size(1), device=x.device, dtype=x.dtype)
+            combine_topk(expanded=expanded, out=output, k=gates.size(1), gates=gates)
+            saved_expanded = expanded
+        ctx.save_for_backward(
+            x, expert_weights, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, saved_expanded
+        )
+        ctx.k, ctx.grouped_in, ctx.grouped_out = k, grouped_in, grouped_out
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, W, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, expanded = ctx.saved_tensors
+        k, grouped_in, grouped_out = ctx.k, ctx.grouped_in, ctx.grouped_out
+        E, K, N = W.shape
+        M = sorted_expert_idxs.size(0)
+        if grad_out.stride(-1) != 1:
+            grad_out = grad_out.contiguous()
+
+        d_gates = None
+        if gates is not None:
+            d_gates = torch.empty_like(gates, memory_format=torch.contiguous_format)
+            gate_grad(expanded=expanded, grad_out=grad_out, d_gates=d_gates)
+
+        # gradient w.r.t. the expanded output, in grouped order
+        if grouped_out:
+            assert gates is None, "gates are applied to scattered outputs"
+            grouped_grad = grad_out
+        else:
+            grouped_grad = torch.empty(M, N, device=x.device, dtype=x.dtype)
+            group(
+                A=grad_out,
+                sorted_expert_idxs=sorted_scattered_idxs,
+                out=grouped_grad,
+                coeff=None if gates is None else gates.flatten(),
+                fan_out=1 if gates is None else gates.size(1),
+            )
+
+        # weight gradient; the token gather of the up-projection is fused into the kernel
+        d_weights = torch.empty_like(W)  # keeps the strides of the view
+        group_bwd_W(
+            DY=grouped_grad,
+            X=x,
+            expert_offsets=expert_offsets,
+            DW=d_weights,
+            E=E,
+            x_index=None if grouped_in else sorted_scattered_idxs,
+            x_fan_out=1 if grouped_in else k,
+        )
+
+        # input gradient: grouped_grad @ W[e]^T, written grouped or scattered
+        d_expanded_input = torch.empty(M, K, device=x.device, dtype=x.dtype)
+        scatter2scatter(
+            X=grouped_grad,
+            W=W.permute(0, 2, 1),
+            sorted_expert_idxs=sorted_expert_idxs,
+            sorted_scattered_idxs=sorted_scattered_idxs,
+            expert_offsets=expert_offsets,
+            out=d_expanded_input,
+            FAN_OUT=1,
+            x_grouped=True,
+            y_grouped=grouped_in,
+        )
+        if k == 1:
+            d_input = d_expanded_input
+        else:
+            d_input = torch.empty_like(x, memory_format=torch.contiguous_format)
+            combine_topk(expanded=d_expanded_input, out=d_input, k=k, gates=None)
+
+        return d_input, d_weights, None, None, None, None, d_gates, None, None
+
+
+def scattered_experts(
+    inputs: torch.Tensor,
+    expert_weights: torch.Tensor,
+    k: int,
+    sorted_expert_idxs: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    gates: torch.Tensor | None = None,
+    grouped_in: bool = False,
+    grouped_out: bool = False,
+) -> torch.Tensor:
+    return _ScatteredExperts.apply(
+        inputs,
+        expert_weights,
+        k,
+        sorted_expert_idxs,
+        sorted_scattered_idxs,
+        expert_offsets,
+        gates,
+        grouped_in,
+        grouped_out,
+    )
+
+
+class _SwigluExperts(torch.autograd.Function):
+    """Both projections with SwiGLU fused; weights in their stored layouts [E, 2I, H] and [E, H, I]."""
+
+    @staticmethod
+    def forward(ctx, x, w_up, w_down, gates, sorted_scattered_idxs, expert_offsets):
+        T, H = x.shape
+        E, I2, _ = w_up.shape
+        k = gates.size(1)
+        M = T * k
+        needs_grad = any(ctx.needs_input_grad)
+        preact = torch.empty(M, I2, device=x.device, dtype=x.dtype) if needs_grad else None
+        act = torch.empty(M, I2 // 2, device=x.device, dtype=x.dtype)
+        up_projection_swiglu(
+            X=x,
+            W=w_up,
+            sorted_scattered_idxs=sorted_scattered_idxs,
+            expert_offsets=expert_offsets,
+            act=act,
+            preact=preact,
+            FAN_OUT=k,
+        )
+        expanded = torch.empty(M, H, device=x.device, dtype=x.dtype)
+        scatter2scatter(
+            X=act,
+            W=w_down.permute(0, 2, 1),
+            sorted_expert_idxs=sorted_scattered_idxs,
+            sorted_scattered_idxs=sorted_scattered_idxs,
+            expert_offsets=expert_offsets,
+            out=expanded,
+            FAN_OUT=1,
+            x_grouped=True,
+            y_grouped=False,
+        )
+        y = torch.empty(T, H, device=x.device, dtype=x.dtype)
+        combine_topk(expanded=expanded, out=y, k=k, gates=gates)
+        if needs_grad:
+            ctx.save_for_backward(x, w_up, w_down, gates, sorted_scattered_idxs, expert_offsets, preact, act, expanded)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, w_up, w_down, gates, idx, expert_offsets, preact, act, expanded = ctx.saved_tensors
+        T, H = x.shape
+        E, I2, _ = w_up.shape
+        k = gates.size(1)
+        M = T * k
+        if grad_out.stride(-1) != 1:
+            grad_out = grad_out.contiguous()
+
+        d_gates = torch.empty_like(gates, memory_format=torch.contiguous_format)
+        gate_grad(expanded=expanded, grad_out=grad_out, d_gates=d_gates)
+
+        grouped_grad = torch.empty(M, H, device=x.device, dtype=x.dtype)
+        group(A=grad_out, sorted_expert_idxs=idx, out=grouped_grad, coeff=gates.flatten(), fan_out=k)
+
+        d_w_down = torch.empty_like(w_down)
+        group_bwd_W(DY=grouped_grad, X=act, expert_offsets=expert_offsets, DW=d_w_down.permute(0, 2, 1), E=E)
+
+        d_preact = torch.empty_like(preact)
+        down_projection_dgrad_swiglu(
+            DY=grouped_grad, W=w_down, preact=preact, expert_offsets=expert_offsets, d_preact=d_preact
+        )
+
+        d_w_up = torch.empty_like(w_up)
+        group_bwd_W(
+            DY=d_preact,
+            X=x,
+            expert_offsets=expert_offsets,
+            DW=d_w_up.permute(0, 2, 1),
+            E=E,
+            x_index=idx,
+            x_fan_out=k,
+        )
+
+        d_expanded = torch.empty(M, H, device=x.device, dtype=x.dtype)
+        scatter2scatter(
+            X=d_preact,
+            W=w_up,
+            sorted_expert_idxs=idx,
+            sorted_scattered_idxs=idx,
+            expert_offsets=expert_offsets,
+            out=d_expanded,
+            FAN_OUT=1,
+            x_grouped=True,
+            y_grouped=False,
+        )
+        d_x = torch.empty_like(x, memory_format=torch.contiguous_format)
+        combine_topk(expanded=d_expanded, out=d_x, k=k, gates=None)
+        return d_x, d_w_up, d_w_down, d_gates, None, None
+
+
+class Experts(XMAModule):
+    """Stacked expert weights [E, out_features, in_features] (xma/layers/moe/__init__.py:23-125)."""
+
+    def __init__(
+        self, num_experts: int, in_features: int, out_features: int, add_bias: bool = True, std: float | None = None
+    ) -> None:
+        super().__init__()
+
+        self.weight = nn.Parameter(torch.empty(num_experts, out_features, in_features))
+        self.bias = nn.Parameter(torch.empty(num_experts, out_features)) if add_bias else None
+
+        self.std = std
+        self.num_experts = num_experts
+        self.in_features = in_features
+        self.out_features = out_features
+
+        # kept so that state_dicts stay interchangeable with the reference's (:41-42)
+        self.register_buffer("N_array", torch.empty((num_experts,), dtype=torch.uint32))
+        self.register_buffer("K_array", torch.empty((num_experts,), dtype=torch.uint32))
+
+        self.reset_parameters()
+
+    def grouped_forward(
+        self,
+        input: torch.Tensor,
+        num_experts_per_token: int,
+        sorted_expert_idxs: torch.Tensor,
+        sorted_scattered_idxs: torch.Tensor,
+        expert_offsets: torch.Tensor,
+        gates: torch.Tensor | None = None,
+        grouped_in: bool = False,
+        grouped_out: bool = False,
+    ) -> torch.Tensor:
+        assert self.bias is None, "the kernel path has no bias support"
+        return scattered_experts(
+            inputs=input,
+            expert_weights=self.weight.permute(0, 2, 1),
+            k=num_experts_per_token,
+            sorted_expert_idxs=sorted_expert_idxs,
+            sorted_scattered_idxs=sorted_scattered_idxs,
+            expert_offsets=expert_offsets,
+            gates=gates,
+            grouped_in=grouped_in,
+            grouped_out=grouped_out,
+        )
+
+    def extra_repr(self) -> str:
+        return f"num_experts={self.num_experts}, in_features={self.in_features}, out_features={self.out_features}"
+
+    @torch.no_grad()
+    def reset_parameters(self) -> None:
+        nn.init.normal_(self.weight, mean=0, std=self.std)
+        if self.bias is not None:
+            self.bias.zero_()
+        self.N_array.fill_(self.out_features)
+        self.K_array.fill_(self.in_features)
+
+
+class MoE(XMAModule):
+    def __init__(
+        self,
+        num_experts: int,
+        num_experts_per_tok: int,
+        hidden_size: int,
+        intermediate_size: int,
+        activation_function: Callable,
+        is_glu: bool,
+        add_bias: bool,
+        std: float,
+    ) -> None:
+        super().__init__()
+
+        self.num_experts = num_experts
+        self.top_k = num_experts_per_tok
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.is_glu = is_glu
+
+        self.gate = nn.Linear(in_features=hidden_size, out_features=num_experts, bias=False)
+        self.c_fc = Experts(
+            num_experts=num_experts,
+            in_features=hidden_size,
+            out_features=2 * intermediate_size if is_glu else intermediate_size,
+            add_bias=add_bias,
+            std=std,
+        )
+        self.act = activation_function
+        self.c_proj = Experts(
+            num_experts=num_experts,
+            in_features=intermediate_size,
+            out_features=hidden_size,
+            add_bias=add_bias,
+            std=std,
+        )
+
+    def forward(
+        self, hidden_states: torch.Tensor, *, kernel_backend: KernelBackend | None = None
+    ) -> tuple[torch.Tensor, torch.Tensor]:
+        """Returns (output with the input's shape, router_logits[tokens, num_experts])."""
+
+        original_shape = hidden_states.shape
+        hidden_states = hidden_states.reshape(-1, self.hidden_size)
+
+        router_logits, router_weights, selected_experts = self._compute_routing_weights(
+            hidden_states, kernel_backend=kernel_backend
+        )
+        hidden_states = self._compute_experts(
+            hidden_states, router_weights, selected_experts, kernel_backend=kernel_backend
+        )
+        return hidden_states.view(original_shape), router_logits
+
+    def _compute_routing_weights(
+        self, hidden_states: torch.Tensor, *, kernel_backend: KernelBackend | None = None
+    ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        router_logits = self.gate(hidden_states)
+        router_weights, selected_experts = topk_softmax(router_logits, self.top_k, kernel_backend=kernel_backend)
+        return router_logits, router_weights, selected_experts
+
+    def _compute_experts(
+        self,
+        hidden_states: torch.Tensor,
+        router_weights: torch.Tensor,
+        selected_experts: torch.Tensor,
+        *,
+        kernel_backend: KernelBackend | None = None,
+    ) -> torch.Tensor:
+        resolve_backend(kernel_backend, "MoE")
+        assert self.c_fc.bias is None and self.c_proj.bias is None, "the kernel path has no bias support"
+
+        routing = route_tokens(selected_experts, self.num_experts)
+
+        if self.act is swiglu_packed and self.is_glu:
+            return _SwigluExperts.apply(
+                hidden_states,
+                self.c_fc.weight,
+                self.c_proj.weight,
+                router_weights,
+                routing.sorted_scattered_idxs,
+                routing.expert_offsets,
+            )
+
+        hidden_states = self.c_fc.grouped_forward(
+            hidden_states,
+            self.top_k,
+            routing.sorted_expert_idxs,
+            routing.sorted_scattered_idxs,
+            routing.expert_offsets,
+            grouped_in=False,
+            grouped_out=True,
+        )
+        hidden_states = self.act(hidden_states)
+        hidden_states = self.c_proj.grouped_forward(
+            hidden_states,
+            1,
+            routing.sorted_expert_idxs,
+            routing.sorted_scattered_idxs,
+            routing.expert_offsets,
+            gates=router_weights,
+            grouped_in=True,
+            grouped_out=False,
+        )
+        return hidden_states

@@ -1,0 +1,551 @@
+"""torch operators (`xma::*`) over the C ABI of libxma_hip.so.
+
+Every operator follows the reference's out-parameter convention (xma/custom_op.py:64-90 and the
+stubs it wraps, e.g. xma/layers/moe/triton_implementation/scatter_kernel.py:137-147): the caller
+allocates outputs with torch, the operator mutates them and returns None, so the native code never
+owns memory.  Names and argument meaning follow the reference operators they replace; where the
+reference has a `_cuda` suffix the operator here ends in `_rocm`.
+
+`expert_offsets` is always the int32 vector of E+1 exclusive prefix sums (leading 0).  The
+reference passes the inclusive cumsum of length E (xma/layers/moe/__init__.py:225); the exclusive
+form is the same data with the implicit 0 stored.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _native as nat
+from .custom_op import xma_op
+
+
+def _i64(t: torch.Tensor | None) -> int:
+    if t is None:
+        return 0
+    if t.dtype == torch.int64:
+        return 1
+    if t.dtype == torch.int32:
+        return 0
+    raise TypeError(f"index tensors must be int32 or int64, got {t.dtype}")
+
+
+def _row_stride(t: torch.Tensor) -> int:
+    """Row stride of a 2-D tensor whose rows are contiguous."""
+
+    assert t.dim() == 2, "expected a 2-D tensor"
+    assert t.size(1) <= 1 or t.stride(1) == 1, "rows must be contiguous"
+    return t.stride(0) if t.size(0) > 1 else max(t.stride(0), t.size(1))
+
+
+def _check_offsets(expert_offsets: torch.Tensor, E: int) -> None:
+    assert expert_offsets.dtype == torch.int32 and expert_offsets.is_contiguous()
+    assert expert_offsets.numel() == E + 1, "expert_offsets must hold E + 1 exclusive prefix sums"
+
+
+# ------------------------------------------------------------------------------------------------
+# routing
+# ------------------------------------------------------------------------------------------------
+@xma_op(mutates_args={"output"})
+def continuous_count_rocm(x: torch.Tensor, output: torch.Tensor, E: int) -> None:
+    """output[e] = number of elements of x equal to e, e in [0, E); replaces continuous_count_cuda."""
+
+    nat.require_device(x, output)
+    assert output.dtype == torch.uint32 and output.numel() == E and output.is_contiguous()
+    x = x.contiguous()
+    nat.call("xma_continuous_count", x.data_ptr(), _i64(x), x.numel(), E, output.data_ptr(), nat.stream())
+
+
+@xma_op(mutates_args={"counts", "expert_offsets", "sorted_expert_idxs", "sorted_scattered_idxs"})
+def route_build_rocm(
+    selected_experts: torch.Tensor,
+    counts: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    sorted_expert_idxs: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    E: int,
+) -> None:
+    """Histogram, exclusive offsets and stable sort permutation of the flattened expert choices."""
+
+    nat.require_device(selected_experts, counts, expert_offsets, sorted_expert_idxs, sorted_scattered_idxs)
+    ids = selected_experts.contiguous().view(-1)
+    n = ids.numel()
+    assert counts.dtype == torch.uint32 and counts.numel() == E and counts.is_contiguous()
+    _check_offsets(expert_offsets, E)
+    assert sorted_expert_idxs.dtype == sorted_scattered_idxs.dtype
+    assert sorted_expert_idxs.numel() == n and sorted_scattered_idxs.numel() == n
+    assert sorted_expert_idxs.is_contiguous() and sorted_scattered_idxs.is_contiguous()
+    ws_bytes = nat.load().xma_route_workspace_bytes(n, E)
+    workspace = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=ids.device)
+    nat.call(
+        "xma_route_build",
+        ids.data_ptr(),
+        _i64(ids),
+        n,
+        E,
+        counts.data_ptr(),
+        expert_offsets.data_ptr(),
+        sorted_expert_idxs.data_ptr(),
+        sorted_scattered_idxs.data_ptr(),
+        _i64(sorted_scattered_idxs),
+        workspace.data_ptr(),
+        workspace.numel(),
+        nat.stream(),
+    )
+
+
+@xma_op(mutates_args={"weights", "indices"})
+def topk_softmax_rocm(logits: torch.Tensor, weights: torch.Tensor, indices: torch.Tensor, k: int) -> None:
+    """Top-k (ties: lower index first) and softmax over the selected logits, one row per token."""
+
+    nat.require_device(logits, weights, indices)
+    assert logits.dim() == 2 and logits.stride(1) == 1
+    T, E = logits.shape
+    assert weights.shape == (T, k) and weights.dtype == logits.dtype and weights.is_contiguous()
+    assert indices.shape == (T, k) and indices.is_contiguous()
+    nat.call(
+        "xma_topk_softmax",
+        logits.data_ptr(),
+        nat.dtype_code(logits),
+        T,
+        E,
+        k,
+        _row_stride(logits),
+        weights.data_ptr(),
+        indices.data_ptr(),
+        _i64(indices),
+        nat.stream(),
+    )
+
+
+@xma_op(mutates_args={"d_logits"})
+def topk_softmax_backward_rocm(
+    logits: torch.Tensor, d_weights: torch.Tensor, indices: torch.Tensor, d_logits: torch.Tensor
+) -> None:
+    nat.require_device(logits, d_weights, indices, d_logits)
+    T, E = logits.shape
+    k = indices.size(1)
+    d_weights = d_weights.contiguous()
+    assert d_logits.shape == (T, E) and d_logits.stride(1) == 1 and d_logits.dtype == logits.dtype
+    assert d_weights.dtype == logits.dtype
+    nat.call(
+        "xma_topk_softmax_bwd",
+        logits.data_ptr(),
+        _row_stride(logits),
+        d_weights.data_ptr(),
+        indices.data_ptr(),
+        _i64(indices),
+        nat.dtype_code(logits),
+        T,
+        E,
+        k,
+        d_logits.data_ptr(),
+        _row_stride(d_logits),
+        nat.stream(),
+    )
+
+
+# ------------------------------------------------------------------------------------------------
+# row moves
+# ------------------------------------------------------------------------------------------------
+@xma_op(mutates_args={"out"})
+def group(
+    A: torch.Tensor,
+    sorted_expert_idxs: torch.Tensor,
+    out: torch.Tensor,
+    coeff: torch.Tensor | None = None,
+    fan_out: int = 1,
+) -> None:
+    """out[p] = A[idx[p] // fan_out] * coeff[idx[p]]; `sorted_expert_idxs` carries the row index
+    table, as in the reference (xma/layers/moe/triton_implementation/group_kernel.py:69-100)."""
+
+    nat.require_device(A, sorted_expert_idxs, out, coeff)
+    assert A.dtype == out.dtype and A.size(1) == out.size(1)
+    idx = sorted_expert_idxs.contiguous()
+    assert out.size(0) == idx.numel()
+    if coeff is not None:
+        coeff = coeff.contiguous()
+        assert coeff.dtype == A.dtype
+    nat.call(
+        "xma_gather_rows",
+        A.data_ptr(),
+        _row_stride(A),
+        out.data_ptr(),
+        _row_stride(out),
+        idx.data_ptr(),
+        _i64(idx),
+        out.size(0),
+        out.size(1),
+        nat.dtype_code(A),
+        fan_out,
+        nat.ptr(coeff),
+        nat.stream(),
+    )
+
+
+@xma_op(mutates_args={"out"})
+def ungroup(A: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> None:
+    """out[index[p]] = A[p]: the inverse row permutation of `group`."""
+
+    nat.require_device(A, index, out)
+    assert A.dtype == out.dtype and A.size(1) == out.size(1) and A.size(0) == index.numel()
+    index = index.contiguous()
+    nat.call(
+        "xma_scatter_rows",
+        A.data_ptr(),
+        _row_stride(A),
+        out.data_ptr(),
+        _row_stride(out),
+        index.data_ptr(),
+        _i64(index),
+        A.size(0),
+        A.size(1),
+        nat.dtype_code(A),
+        nat.stream(),
+    )
+
+
+@xma_op(mutates_args={"out"})
+def combine_topk(expanded: torch.Tensor, out: torch.Tensor, k: int, gates: torch.Tensor | None = None) -> None:
+    """out[t] = sum_j gates[t, j] * expanded[t*k + j] (plain sum when gates is None)."""
+
+    nat.require_device(expanded, out, gates)
+    T = out.size(0)
+    assert expanded.size(0) == T * k and expanded.size(1) == out.size(1) and expanded.dtype == out.dtype
+    if gates is not None:
+        gates = gates.contiguous()
+        assert gates.numel() == T * k and gates.dtype == out.dtype
+    nat.call(
+        "xma_combine_topk",
+        expanded.data_ptr(),
+        _row_stride(expanded),
+        nat.ptr(gates),
+        out.data_ptr(),
+        _row_stride(out),
+        T,
+        k,
+        out.size(1),
+        nat.dtype_code(out),
+        nat.stream(),
+    )
+
+
+@xma_op(mutates_args={"d_gates"})
+def gate_grad(expanded: torch.Tensor, grad_out: torch.Tensor, d_gates: torch.Tensor) -> None:
+    """d_gates[t, j] = <expanded[t*k + j], grad_out[t]>."""
+
+    nat.require_device(expanded, grad_out, d_gates)
+    T, k = d_gates.shape
+    assert d_gates.is_contiguous() and d_gates.dtype == expanded.dtype == grad_out.dtype
+    assert expanded.size(0) == T * k and grad_out.size(0) == T and expanded.size(1) == grad_out.size(1)
+    nat.call(
+        "xma_gate_grad",
+        expanded.data_ptr(),
+        _row_stride(expanded),
+        grad_out.data_ptr(),
+        _row_stride(grad_out),
+        d_gates.data_ptr(),
+        T,
+        k,
+        expanded.size(1),
+        nat.dtype_code(expanded),
+        nat.stream(),
+    )
+
+
+# ------------------------------------------------------------------------------------------------
+# swiglu
+# ------------------------------------------------------------------------------------------------
+@xma_op(mutates_args={"y"})
+def swiglu_forward_rocm(g: torch.Tensor, u: torch.Tensor, y: torch.Tensor) -> None:
+    nat.require_device(g, u, y)
+    assert g.shape == u.shape == y.shape and g.dtype == u.dtype == y.dtype
+    rows, cols = g.shape
+    nat.call(
+        "xma_swiglu_forward",
+        g.data_ptr(),
+        _row_stride(g),
+        u.data_ptr(),
+        _row_stride(u),
+        y.data_ptr(),
+        _row_stride(y),
+        rows,
+        cols,
+        nat.dtype_code(g),
+        nat.stream(),
+    )
+
+
+@xma_op(mutates_args={"dg", "du"})
+def swiglu_backward_rocm(
+    g: torch.Tensor, u: torch.Tensor, dy: torch.Tensor, dg: torch.Tensor, du: torch.Tensor
+) -> None:
+    nat.require_device(g, u, dy, dg, du)
+    assert g.shape == u.shape == dy.shape == dg.shape == du.shape
+    assert g.dtype == u.dtype == dy.dtype == dg.dtype == du.dtype
+    rows, cols = g.shape
+    nat.call(
+        "xma_swiglu_backward",
+        g.data_ptr(),
+        _row_stride(g),
+        u.data_ptr(),
+        _row_stride(u),
+        dy.data_ptr(),
+        _row_stride(dy),
+        dg.data_ptr(),
+        _row_stride(dg),
+        du.data_ptr(),
+        _row_stride(du),
+        rows,
+        cols,
+        nat.dtype_code(g),
+        nat.stream(),
+    )
+
+
+# ------------------------------------------------------------------------------------------------
+# grouped GEMM
+# ------------------------------------------------------------------------------------------------
+def _grouped_gemm(
+    *,
+    kind: int,
+    epilogue: int,
+    E: int,
+    rows: int,
+    n: int,
+    k: int,
+    a: torch.Tensor,
+    lda: int,
+    b: torch.Tensor,
+    ldb: int,
+    b_expert_stride: int,
+    c: torch.Tensor,
+    ldc: int,
+    c_expert_stride: int,
+    expert_offsets: torch.Tensor,
+    aux: torch.Tensor | None = None,
+    ld_aux: int = 0,
+    in_index: torch.Tensor | None = None,
+    in_fan_out: int = 1,
+    out_index: torch.Tensor | None = None,
+) -> None:
+    nat.require_device(a, b, c, aux, expert_offsets, in_index, out_index)
+    _check_offsets(expert_offsets, E)
+    if in_index is not None and out_index is not None:
+        assert in_index.dtype == out_index.dtype
+    index = in_index if in_index is not None else out_index
+    args = nat.GroupedGemmArgs()
+    args.kind, args.dtype, args.epilogue, args.num_experts = kind, nat.dtype_code(a), epilogue, E
+    args.rows, args.n, args.k = rows, n, k
+    args.a, args.lda = a.data_ptr(), lda
+    args.b, args.ldb, args.b_expert_stride = b.data_ptr(), ldb, b_expert_stride
+    args.c, args.ldc, args.c_expert_stride = c.data_ptr(), ldc, c_expert_stride
+    args.aux, args.ld_aux = nat.ptr(aux), ld_aux
+    args.expert_offsets = expert_offsets.data_ptr()
+    args.in_index, args.out_index = nat.ptr(in_index), nat.ptr(out_index)
+    args.idx_is_i64, args.in_fan_out = _i64(index), in_fan_out
+    workspace = None
+    if kind != nat.GEMM_MT:
+        ws_bytes = nat.load().xma_grouped_gemm_workspace_bytes(E, rows)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
+        args.workspace, args.workspace_bytes = workspace.data_ptr(), ws_bytes
+    nat.call("xma_grouped_gemm", ctypes.byref(args), nat.stream())
+
+
+def _weight_layout(W: torch.Tensor) -> tuple[int, int]:
+    """(kind, row stride) of a logical [E, K, N] weight tensor from its strides."""
+
+    assert W.dim() == 3
+    if W.stride(1) == 1 and (W.size(2) == 1 or W.stride(2) >= W.size(1)):
+        return nat.GEMM_TN, W.stride(2)  # stored [E, N, K]
+    if W.stride(2) == 1 and (W.size(1) == 1 or W.stride(1) >= W.size(2)):
+        return nat.GEMM_NN, W.stride(1)  # stored [E, K, N]
+    raise ValueError(f"expert weights need one unit stride among the last two dims, got strides {W.stride()}")
+
+
+@xma_op(mutates_args={"out"})
+def scatter2scatter(
+    X: torch.Tensor,
+    W: torch.Tensor,
+    sorted_expert_idxs: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    out: torch.Tensor,
+    FAN_OUT: int,
+    x_grouped: bool = False,
+    y_grouped: bool = False,
+) -> None:
+    """out[o(p)] = X[i(p)] @ W[e(p)] over the grouped positions p.
+
+    i(p) = p if x_grouped else idx[p] // FAN_OUT; o(p) = p if y_grouped else idx[p]
+    (xma/layers/moe/triton_implementation/scatter_kernel.py:105-108,128-131).  W is the logical
+    [E, K, N] tensor; a permuted view of [E, N, K] storage is read in place.
+    """
+
+    assert sorted_scattered_idxs.size(0) == sorted_expert_idxs.size(0)
+    assert sorted_scattered_idxs.size(0) == X.size(0) * FAN_OUT
+    assert out.size(0) == sorted_expert_idxs.size(0)
+    assert out.size(1) == W.size(-1)
+    assert X.size(1) == W.size(1) and X.dtype == W.dtype == out.dtype
+    kind, ldb = _weight_layout(W)
+    idx = sorted_scattered_idxs.contiguous()
+    _grouped_gemm(
+        kind=kind,
+        epilogue=nat.EPI_NONE,
+        E=W.size(0),
+        rows=idx.size(0),
+        n=W.size(2),
+        k=W.size(1),
+        a=X,
+        lda=_row_stride(X),
+        b=W,
+        ldb=ldb,
+        b_expert_stride=W.stride(0),
+        c=out,
+        ldc=_row_stride(out),
+        c_expert_stride=0,
+        expert_offsets=expert_offsets,
+        in_index=None if x_grouped else idx,
+        in_fan_out=FAN_OUT,
+        out_index=None if y_grouped else idx,
+    )
+
+
+@xma_op(mutates_args={"DW"})
+def group_bwd_W(
+    DY: torch.Tensor,
+    X: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    DW: torch.Tensor,
+    E: int,
+    x_index: torch.Tensor | None = None,
+    x_fan_out: int = 1,
+) -> None:
+    """DW[e] = X_e^T @ DY_e over expert e's rows; every DW[e] is written (zeros for empty experts).
+
+    DW is the logical [E, K, N] gradient (K = X columns, N = DY columns) with the strides of the
+    weight view it belongs to (xma/layers/moe/triton_implementation/group_backward_kernel.py:102-125).
+    With `x_index`, row p of X is read from X[x_index[p] // x_fan_out] (fused token gather).
+    """
+
+    assert DW.dim() == 3 and DW.size(0) == E and DW.size(1) == X.size(1) and DW.size(2) == DY.size(1)
+    assert DY.dtype == X.dtype == DW.dtype
+    rows = DY.size(0)
+    if x_index is not None:
+        x_index = x_index.contiguous()
+        assert x_index.numel() == rows
+    else:
+        assert X.size(0) == rows
+    common = dict(
+        kind=nat.GEMM_MT,
+        epilogue=nat.EPI_NONE,
+        E=E,
+        rows=rows,
+        b_expert_stride=0,
+        c=DW,
+        c_expert_stride=DW.stride(0),
+        expert_offsets=expert_offsets,
+    )
+    if DW.stride(1) == 1:  # storage [E, N, K]: rows of C[e] come from DY, columns from X
+        _grouped_gemm(
+            n=DY.size(1),
+            k=X.size(1),
+            a=DY,
+            lda=_row_stride(DY),
+            b=X,
+            ldb=_row_stride(X),
+            ldc=DW.stride(2),
+            in_index=x_index,
+            in_fan_out=x_fan_out,
+            **common,
+        )
+    elif DW.stride(2) == 1:  # storage [E, K, N]: rows of C[e] come from X
+        if x_index is not None:
+            gathered = torch.empty(rows, X.size(1), dtype=X.dtype, device=X.device)
+            group(X, x_index, gathered, None, x_fan_out)
+            X = gathered
+        _grouped_gemm(
+            n=X.size(1),
+            k=DY.size(1),
+            a=X,
+            lda=_row_stride(X),
+            b=DY,
+            ldb=_row_stride(DY),
+            ldc=DW.stride(1),
+            **common,
+        )
+    else:
+        raise ValueError(f"DW needs one unit stride among the last two dims, got strides {DW.stride()}")
+
+
+@xma_op(mutates_args={"act", "preact"})
+def up_projection_swiglu(
+    X: torch.Tensor,
+    W: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    act: torch.Tensor,
+    preact: torch.Tensor | None,
+    FAN_OUT: int,
+) -> None:
+    """act[p] = swiglu_packed(X[idx[p] // FAN_OUT] @ W[e(p)]^T) with W stored [E, 2I, H] (up rows
+    first, gate rows second); `preact`, when given, receives the [M, 2I] product for backward."""
+
+    E, N, K = W.shape
+    assert W.is_contiguous() and X.size(1) == K and act.size(1) * 2 == N
+    idx = sorted_scattered_idxs.contiguous()
+    _grouped_gemm(
+        kind=nat.GEMM_TN,
+        epilogue=nat.EPI_SWIGLU,
+        E=E,
+        rows=idx.size(0),
+        n=N,
+        k=K,
+        a=X,
+        lda=_row_stride(X),
+        b=W,
+        ldb=K,
+        b_expert_stride=N * K,
+        c=act,
+        ldc=_row_stride(act),
+        c_expert_stride=0,
+        expert_offsets=expert_offsets,
+        aux=preact,
+        ld_aux=0 if preact is None else _row_stride(preact),
+        in_index=idx,
+        in_fan_out=FAN_OUT,
+    )
+
+
+@xma_op(mutates_args={"d_preact"})
+def down_projection_dgrad_swiglu(
+    DY: torch.Tensor,
+    W: torch.Tensor,
+    preact: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    d_preact: torch.Tensor,
+) -> None:
+    """d_preact = swiglu_packed'(preact) applied to (DY_grouped @ W[e]) with W stored [E, H, I]."""
+
+    E, H, I = W.shape
+    assert W.is_contiguous() and DY.size(1) == H and preact.size(1) == 2 * I and d_preact.shape == preact.shape
+    _grouped_gemm(
+        kind=nat.GEMM_NN,
+        epilogue=nat.EPI_SWIGLU_BWD,
+        E=E,
+        rows=DY.size(0),
+        n=I,
+        k=H,
+        a=DY,
+        lda=_row_stride(DY),
+        b=W,
+        ldb=I,
+        b_expert_stride=H * I,
+        c=d_preact,
+        ldc=_row_stride(d_preact),
+        c_expert_stride=0,
+        expert_offsets=expert_offsets,
+        aux=preact,
+        ld_aux=_row_stride(preact),
+    )
