@@ -1,0 +1,202 @@
+"""Benchmark of the MoE hot path on one MI355X.
+
+A "step" is one forward + backward pass of the Mixtral-shaped MoE layer (bf16 with fp32
+accumulation, hidden 4096, per-expert intermediate 14336, 8 experts, top-2, 8192 tokens) over
+synthetic inputs that are already resident in HBM.  Prints ONE JSON line with the whole-job
+throughput in tokens/s, the roofline position of the dominant kernel (timed with events on the
+launch stream during the timed steps) and a CPU baseline: the torch restatement of the
+reference's torch path (oracle/torch_oracle.py) timed on this host's cores on a bounded sample.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published peaks (dense)
+PEAK_BF16_FLOPS = 2.5e15
+PEAK_HBM_BYTES = 8.0e12
+
+WORKLOAD = {
+    "workload": "Mixtral-shaped MoE layer, forward+backward",
+    "tokens": 8192,
+    "hidden": 4096,
+    "intermediate": 14336,
+    "experts": 8,
+    "top_k": 2,
+    "activation": "swiglu_packed",
+    "routing": "linear gate, near-uniform expert load",
+}
+
+
+def _parse() -> argparse.Namespace:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    return ap.parse_args()
+
+
+def _cpu_baseline(moe, x, d_y, sample_tokens: int) -> dict:
+    """Reference torch path on the host cores, same layer, first `sample_tokens` tokens."""
+
+    import torch
+
+    from oracle import torch_oracle as to
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    k = moe.top_k
+    params = [p.detach().cpu().requires_grad_() for p in (moe.gate.weight, moe.c_fc.weight, moe.c_proj.weight)]
+    xs = x.detach()[:sample_tokens].cpu().requires_grad_()
+    dys = d_y[:sample_tokens].cpu()
+
+    def step() -> float:
+        t0 = time.perf_counter()
+        y, _ = to.moe_forward(xs, params[0], params[1], params[2], k)
+        y.backward(dys)
+        dt = time.perf_counter() - t0
+        xs.grad = None
+        for p in params:
+            p.grad = None
+        return dt
+
+    step()  # warm-up
+    seconds = step()
+    return {
+        "value": sample_tokens / seconds,
+        "unit": "tokens/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"first {sample_tokens} of {x.size(0)} tokens of the same layer and dtype, forward+backward, "
+        f"1 timed iteration after 1 warm-up ({seconds:.2f} s); per-expert weight-gradient zero fills do not "
+        "shrink with the sample, so the full-size rate is no lower than this",
+    }
+
+
+def main() -> int:
+    args = _parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import flash_model_architectures_amd as xma
+    from flash_model_architectures_amd import _native
+
+    _native.load()  # fail loudly if the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    T, H, I = WORKLOAD["tokens"], WORKLOAD["hidden"], WORKLOAD["intermediate"]
+    E, k = WORKLOAD["experts"], WORKLOAD["top_k"]
+    dt = torch.bfloat16
+
+    moe = xma.MoE(E, k, H, I, xma.swiglu_packed, True, False, 0.02).to(dt).to(dev)
+    x = torch.randn(T, H, device=dev).to(dt).requires_grad_()
+    d_y = torch.randn(T, H, device=dev).to(dt)
+
+    def step() -> None:
+        y, _ = moe(x)
+        y.backward(d_y)
+        x.grad = None
+        moe.zero_grad(set_to_none=True)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    timeline = _native.Timeline()
+    _native.set_timeline(timeline)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    _native.set_timeline(None)
+
+    ms_per_step = seconds / args.steps * 1e3
+    tokens_per_s = T * args.steps / seconds
+    gemm_flops = 18.0 * T * k * H * I  # forward 6*M*H*I, backward twice that
+
+    kernels = []
+    for tag, row in sorted(timeline.summary().items(), key=lambda kv: -kv[1]["ms"]):
+        avg_ms = row["ms"] / row["launches"]
+        entry = {
+            "kernel": tag,
+            "launches_per_step": row["launches"] / args.steps,
+            "avg_ms": round(avg_ms, 4),
+            "ms_per_step": round(row["ms"] / args.steps, 4),
+        }
+        if row["flops"] > 0:
+            entry["tflops"] = round(row["flops"] / row["ms"] / 1e9, 2)
+            entry["frac_of_bf16_peak"] = round(row["flops"] / (row["ms"] * 1e-3) / PEAK_BF16_FLOPS, 4)
+        elif row["bytes"] > 0:
+            entry["gbps"] = round(row["bytes"] / row["ms"] / 1e6, 1)
+            entry["frac_of_hbm_peak"] = round(row["bytes"] / (row["ms"] * 1e-3) / PEAK_HBM_BYTES, 4)
+        kernels.append(entry)
+
+    dominant = kernels[0]
+    if "tflops" in dominant:
+        roofline = {
+            "kernel": dominant["kernel"],
+            "bound": "mfma",
+            "achieved": dominant["tflops"],
+            "peak": PEAK_BF16_FLOPS / 1e12,
+            "unit": "TFLOP/s",
+            "frac": dominant["frac_of_bf16_peak"],
+            "traffic": None,
+        }
+    else:
+        roofline = {
+            "kernel": dominant["kernel"],
+            "bound": "hbm",
+            "achieved": dominant.get("gbps", 0.0),
+            "peak": PEAK_HBM_BYTES / 1e9,
+            "unit": "GB/s",
+            "frac": dominant.get("frac_of_hbm_peak", 0.0),
+            "traffic": None,
+        }
+
+    gemm_ms = sum(kr["ms_per_step"] for kr in kernels if kr["kernel"].startswith("xma_grouped_gemm"))
+    result = {
+        "metric": "MoE fwd+bwd tokens/s (Mixtral-shaped bf16 layer, 1 GPU)",
+        "value": round(tokens_per_s, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": WORKLOAD,
+        "layer_tflops": round(gemm_flops / (ms_per_step * 1e-3) / 1e12, 2),
+        "grouped_gemm_tflops": round(gemm_flops / (gemm_ms * 1e-3) / 1e12, 2) if gemm_ms > 0 else None,
+        "grouped_gemm_frac_of_bf16_peak": round(gemm_flops / (gemm_ms * 1e-3) / PEAK_BF16_FLOPS, 4) if gemm_ms else None,
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = _cpu_baseline(moe, x, d_y, args.cpu_sample_tokens)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

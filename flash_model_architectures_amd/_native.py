@@ -148,10 +148,47 @@ def last_error() -> str:
     return load().xma_last_error().decode()
 
 
-def call(name: str, *args) -> None:
+class Timeline:
+    """Optional per-call timing: brackets every native call with events on the launch stream and
+    remembers the algorithmic work (FLOPs, bytes) the caller attributes to it."""
+
+    def __init__(self) -> None:
+        self.records: list[tuple[str, torch.cuda.Event, torch.cuda.Event, float, float]] = []
+
+    def summary(self) -> dict[str, dict[str, float]]:
+        """tag -> launches, total milliseconds, FLOPs and bytes (synchronises the device)."""
+
+        torch.cuda.synchronize()
+        out: dict[str, dict[str, float]] = {}
+        for tag, start, end, flops, nbytes in self.records:
+            row = out.setdefault(tag, {"launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0})
+            row["launches"] += 1
+            row["ms"] += start.elapsed_time(end)
+            row["flops"] += flops
+            row["bytes"] += nbytes
+        return out
+
+
+_timeline: Timeline | None = None
+
+
+def set_timeline(timeline: Timeline | None) -> None:
+    global _timeline
+    _timeline = timeline
+
+
+def call(name: str, *args, tag: str | None = None, flops: float = 0.0, nbytes: float = 0.0) -> None:
     """Invoke an int-returning entry point and turn a non-zero status into RuntimeError."""
 
-    status = getattr(load(), name)(*args)
+    fn = getattr(load(), name)
+    if _timeline is None:
+        status = fn(*args)
+    else:
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        status = fn(*args)
+        end.record()
+        _timeline.records.append((tag or name, start, end, flops, nbytes))
     if status != 0:
         raise RuntimeError(f"{name} failed: {last_error()}")
 

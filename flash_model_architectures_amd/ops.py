@@ -54,7 +54,16 @@ def continuous_count_rocm(x: torch.Tensor, output: torch.Tensor, E: int) -> None
     nat.require_device(x, output)
     assert output.dtype == torch.uint32 and output.numel() == E and output.is_contiguous()
     x = x.contiguous()
-    nat.call("xma_continuous_count", x.data_ptr(), _i64(x), x.numel(), E, output.data_ptr(), nat.stream())
+    nat.call(
+        "xma_continuous_count",
+        x.data_ptr(),
+        _i64(x),
+        x.numel(),
+        E,
+        output.data_ptr(),
+        nat.stream(),
+        nbytes=x.numel() * x.element_size() + 4 * E,
+    )
 
 
 @xma_op(mutates_args={"counts", "expert_offsets", "sorted_expert_idxs", "sorted_scattered_idxs"})
@@ -92,6 +101,7 @@ def route_build_rocm(
         workspace.data_ptr(),
         workspace.numel(),
         nat.stream(),
+        nbytes=n * ids.element_size() + 2 * n * sorted_scattered_idxs.element_size(),
     )
 
 
@@ -181,6 +191,7 @@ def group(
         fan_out,
         nat.ptr(coeff),
         nat.stream(),
+        nbytes=2 * out.numel() * out.element_size() + idx.numel() * idx.element_size(),
     )
 
 
@@ -203,6 +214,7 @@ def ungroup(A: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> None:
         A.size(1),
         nat.dtype_code(A),
         nat.stream(),
+        nbytes=2 * A.numel() * A.element_size() + index.numel() * index.element_size(),
     )
 
 
@@ -228,6 +240,8 @@ def combine_topk(expanded: torch.Tensor, out: torch.Tensor, k: int, gates: torch
         out.size(1),
         nat.dtype_code(out),
         nat.stream(),
+        tag="xma_combine_topk" if gates is not None else "xma_combine_topk(fold)",
+        nbytes=(expanded.numel() + out.numel() + (0 if gates is None else gates.numel())) * out.element_size(),
     )
 
 
@@ -251,6 +265,7 @@ def gate_grad(expanded: torch.Tensor, grad_out: torch.Tensor, d_gates: torch.Ten
         expanded.size(1),
         nat.dtype_code(expanded),
         nat.stream(),
+        nbytes=(expanded.numel() + grad_out.numel() + d_gates.numel()) * expanded.element_size(),
     )
 
 
@@ -274,6 +289,7 @@ def swiglu_forward_rocm(g: torch.Tensor, u: torch.Tensor, y: torch.Tensor) -> No
         cols,
         nat.dtype_code(g),
         nat.stream(),
+        nbytes=3 * rows * cols * g.element_size(),
     )
 
 
@@ -301,6 +317,7 @@ def swiglu_backward_rocm(
         cols,
         nat.dtype_code(g),
         nat.stream(),
+        nbytes=5 * rows * cols * g.element_size(),
     )
 
 
@@ -350,7 +367,8 @@ def _grouped_gemm(
         ws_bytes = nat.load().xma_grouped_gemm_workspace_bytes(E, rows)
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
         args.workspace, args.workspace_bytes = workspace.data_ptr(), ws_bytes
-    nat.call("xma_grouped_gemm", ctypes.byref(args), nat.stream())
+    tag = "xma_grouped_gemm/" + ("TN", "NN", "MT")[kind] + ("", "+swiglu", "+swiglu_bwd")[epilogue]
+    nat.call("xma_grouped_gemm", ctypes.byref(args), nat.stream(), tag=tag, flops=2.0 * rows * n * k)
 
 
 def _weight_layout(W: torch.Tensor) -> tuple[int, int]:

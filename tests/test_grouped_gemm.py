@@ -1,0 +1,158 @@
+"""The ragged GEMM entry point in all three operand layouts and both fused epilogues, against
+per-expert fp32 matmuls on the CPU (the computation `Experts.torch_forward` performs,
+xma/layers/moe/__init__.py:103-106, and its transposes for the gradients)."""
+
+import pytest
+import torch
+
+from flash_model_architectures_amd import ops
+from oracle import torch_oracle as to
+
+from .helpers import TOL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _routing(T, E, k, seed, empty=()):
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn(T, E, generator=g)
+    for e in empty:
+        logits[:, e] = -1e9
+    _, sel = to.routing_weights(logits, k)
+    return to.route(sel, E)
+
+
+def _per_expert(off, fn):
+    return torch.cat([fn(e, slice(off[e], off[e + 1])) for e in range(len(off) - 1)])
+
+
+CASES = [
+    # T, H, I, E, k, empty experts
+    (64, 64, 32, 4, 2, ()),
+    (300, 128, 72, 1, 1, ()),  # one expert: a plain dense GEMM
+    (7, 576, 256, 128, 8, ()),  # the reference's small-batch shape: most experts empty
+    (1000, 576, 264, 32, 4, (2, 31)),  # K tail (264 = 4*64 + 8), N not a tile multiple
+    (2048, 1024, 512, 8, 2, (0,)),
+    (513, 200, 104, 5, 3, (4,)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", CASES)
+def test_all_layouts_and_epilogues(case, dtype):
+    T, H, I, E, k, empty = case
+    tol = TOL[dtype]
+    g = torch.Generator().manual_seed(T + H + I + E)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    w1 = (torch.randn(E, 2 * I, H, generator=g) * 0.05).to(dtype)
+    w2 = (torch.randn(E, H, I, generator=g) * 0.05).to(dtype)
+    r = _routing(T, E, k, T + E, empty)
+    idx, off = r.sorted_scattered_idxs, r.expert_offsets.tolist()
+    M = T * k
+    dev = "cuda"
+    xd, w1d, w2d = x.to(dev), w1.to(dev), w2.to(dev)
+    idxd, offd, sed = idx.to(dev).int(), r.expert_offsets.to(dev), r.sorted_expert_idxs.to(dev).int()
+    xg = x[idx // k].float()
+
+    # TN with row gather: h = x[idx // k] @ W1[e]^T, grouped output
+    h = torch.empty(M, 2 * I, dtype=dtype, device=dev)
+    ops.scatter2scatter(xd, w1d.permute(0, 2, 1), sed, idxd, offd, h, k, False, True)
+    h_ref = _per_expert(off, lambda e, s: xg[s] @ w1[e].float().T)
+    assert_close(h, h_ref, tol, "up projection")
+
+    # TN + SwiGLU epilogue
+    act = torch.empty(M, I, dtype=dtype, device=dev)
+    pre = torch.empty(M, 2 * I, dtype=dtype, device=dev)
+    ops.up_projection_swiglu(xd, w1d, idxd, offd, act, pre, k)
+    assert torch.equal(pre, h)  # same kernel body, same rounding
+    assert_close(act, to.swiglu_packed(h.cpu()), tol, "fused swiglu")
+    act2 = torch.empty_like(act)
+    ops.up_projection_swiglu(xd, w1d, idxd, offd, act2, None, k)  # inference: no pre-activation
+    assert torch.equal(act2, act)
+
+    # TN with row scatter: y_exp[idx[p]] = act[p] @ W2[e]^T
+    y_exp = torch.full((M, H), float("nan"), dtype=dtype, device=dev)
+    ops.scatter2scatter(act, w2d.permute(0, 2, 1), sed, idxd, offd, y_exp, 1, True, False)
+    a32 = act.float().cpu()
+    y_ref = torch.empty(M, H)
+    y_ref[idx] = _per_expert(off, lambda e, s: a32[s] @ w2[e].float().T)
+    assert_close(y_exp, y_ref, tol, "down projection")
+
+    # NN: dA = dY_grouped @ W2[e]
+    dyg = torch.randn(M, H, generator=g).to(dtype)
+    dygd = dyg.to(dev)
+    d_act = torch.empty(M, I, dtype=dtype, device=dev)
+    ops.scatter2scatter(dygd, w2d, sed, idxd, offd, d_act, 1, True, True)
+    d_act_ref = _per_expert(off, lambda e, s: dyg[s].float() @ w2[e].float())
+    assert_close(d_act, d_act_ref, tol, "input gradient")
+
+    # NN + SwiGLU backward epilogue
+    d_pre = torch.empty(M, 2 * I, dtype=dtype, device=dev)
+    ops.down_projection_dgrad_swiglu(dygd, w2d, pre, offd, d_pre)
+    pc = pre.cpu()
+    dg, du = to.swiglu_backward(pc[:, I:], pc[:, :I], d_act.cpu())
+    assert_close(d_pre, torch.cat([du, dg], -1), tol, "fused swiglu backward")
+
+    # NN with row scatter: dXe[idx[p]] = d_pre[p] @ W1[e]
+    d_xe = torch.empty(M, H, dtype=dtype, device=dev)
+    ops.scatter2scatter(d_pre, w1d, sed, idxd, offd, d_xe, 1, True, False)
+    dp = d_pre.float().cpu()
+    d_xe_ref = torch.empty(M, H)
+    d_xe_ref[idx] = _per_expert(off, lambda e, s: dp[s] @ w1[e].float())
+    assert_close(d_xe, d_xe_ref, tol, "scattered input gradient")
+
+    # MT with fused token gather: dW1[e] = d_pre_e^T @ x[idx // k]_e; empty experts must be zero-filled
+    d_w1 = torch.full((E, 2 * I, H), float("nan"), dtype=dtype, device=dev)
+    ops.group_bwd_W(d_pre, xd, offd, d_w1.permute(0, 2, 1), E, idxd, k)
+    d_w1_ref = torch.stack([dp[off[e] : off[e + 1]].T @ xg[off[e] : off[e + 1]] for e in range(E)])
+    assert_close(d_w1, d_w1_ref, tol, "up weight gradient")
+    for e in range(E):
+        if off[e] == off[e + 1]:
+            assert bool(torch.all(d_w1[e] == 0)), f"empty expert {e} not zeroed"
+
+    # MT plain: dW2[e] = dY_e^T @ act_e, and the transposed storage order
+    d_w2 = torch.full((E, H, I), float("nan"), dtype=dtype, device=dev)
+    ops.group_bwd_W(dygd, act, offd, d_w2.permute(0, 2, 1), E)
+    d_w2_ref = torch.stack([dyg[off[e] : off[e + 1]].float().T @ a32[off[e] : off[e + 1]] for e in range(E)])
+    assert_close(d_w2, d_w2_ref, tol, "down weight gradient")
+    d_w2_t = torch.empty(E, I, H, dtype=dtype, device=dev)
+    ops.group_bwd_W(dygd, act, offd, d_w2_t, E)
+    assert_close(d_w2_t, d_w2_ref.transpose(1, 2), tol, "down weight gradient, [E, K, N] storage")
+
+
+def test_argument_validation():
+    dev = "cuda"
+    x = torch.randn(8, 64, device=dev, dtype=torch.bfloat16)
+    w = torch.randn(2, 32, 64, device=dev, dtype=torch.bfloat16)
+    idx = torch.arange(8, device=dev, dtype=torch.int32)
+    se = torch.zeros(8, device=dev, dtype=torch.int32)
+    off = torch.tensor([0, 8, 8], device=dev, dtype=torch.int32)
+    out = torch.empty(8, 32, device=dev, dtype=torch.bfloat16)
+    ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, off, out, 1, False, True)  # sanity: valid call
+    with pytest.raises(RuntimeError, match="multiples"):
+        bad_w = torch.randn(2, 12, 64, device=dev, dtype=torch.bfloat16)
+        ops.scatter2scatter(x, bad_w.permute(0, 2, 1), se, idx, off, out[:, :12], 1, False, True)
+    with pytest.raises(RuntimeError, match="aligned"):
+        shifted = torch.randn(8 * 64 + 8, device=dev, dtype=torch.bfloat16)[1 : 1 + 8 * 64].view(8, 64)
+        ops.scatter2scatter(shifted, w.permute(0, 2, 1), se, idx, off, out, 1, False, True)
+    with pytest.raises(AssertionError):
+        ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, off[:2], out, 1, False, True)
+    with pytest.raises(ValueError):
+        ops.scatter2scatter(x[:, :32], w.permute(0, 2, 1)[:, ::2, ::2], se, idx, off, out[:, :16], 1, False, True)
+
+
+def test_ragged_tail_rows_are_not_touched():
+    """Rows of other experts that share an output tile must keep their values."""
+
+    dev = "cuda"
+    T, H, N, E = 300, 64, 256, 3
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(E, N, H, generator=g) * 0.1).to(torch.bfloat16).to(dev)
+    off = torch.tensor([0, 1, 1, 300], dtype=torch.int32, device=dev)  # sizes 1, 0, 299
+    idx = torch.arange(T, dtype=torch.int32, device=dev)
+    se = torch.cat([torch.zeros(1), torch.full((299,), 2)]).int().to(dev)
+    out = torch.empty(T, N, dtype=torch.bfloat16, device=dev)
+    ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, off, out, 1, True, True)
+    ref = torch.cat([x[:1].float() @ w[0].float().T, x[1:].float() @ w[2].float().T])
+    assert_close(out, ref, TOL[torch.bfloat16])

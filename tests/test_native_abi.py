@@ -1,0 +1,146 @@
+"""Host-side checks that need no GPU: the C ABI's symbol table, the loader, argument validation,
+the Python surface that mirrors the reference, and loud failure off-device."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import flash_model_architectures_amd as xma
+from flash_model_architectures_amd import _native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "xma_hip.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(xma_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared_symbols()
+    for required in [
+        "xma_continuous_count",
+        "xma_route_build",
+        "xma_topk_softmax",
+        "xma_topk_softmax_bwd",
+        "xma_gather_rows",
+        "xma_scatter_rows",
+        "xma_combine_topk",
+        "xma_gate_grad",
+        "xma_swiglu_forward",
+        "xma_swiglu_backward",
+        "xma_grouped_gemm",
+        "xma_last_error",
+    ]:
+        assert required in names
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    assert _native.is_built(), "build the library first: python -m flash_model_architectures_amd.build"
+    lib = ctypes.CDLL(_native.library_path())
+    for name in _declared_symbols():
+        assert hasattr(lib, name), f"{name} is declared in include/xma_hip.h but not exported"
+    assert sorted(_native.PROTOTYPES) == _declared_symbols()  # the Python binding covers the header exactly
+
+
+def test_identification_and_error_channel():
+    lib = _native.load()
+    assert lib.xma_target_arch() == b"gfx950"
+    assert lib.xma_version().decode().count(".") == 2
+    # argument validation happens on the host before any launch, so it is testable without a GPU
+    counts = (ctypes.c_uint32 * 4)()
+    rc = lib.xma_continuous_count(None, 0, 0, 0, counts, None)
+    assert rc != 0 and "bins" in _native.last_error()
+    rc = lib.xma_topk_softmax(None, 2, 4, 8, 9, 8, None, None, 0, None)
+    assert rc != 0 and "k=" in _native.last_error()
+    args = _native.GroupedGemmArgs()
+    args.kind, args.dtype, args.num_experts = 0, 2, 0
+    assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "num_experts" in _native.last_error()
+    args.num_experts, args.n, args.k = 4, 12, 64  # n not a multiple of 8
+    off = (ctypes.c_int32 * 5)()
+    args.expert_offsets = ctypes.cast(off, ctypes.c_void_p)
+    assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "multiples" in _native.last_error()
+    assert lib.xma_grouped_gemm(None, None) != 0
+    assert lib.xma_route_workspace_bytes(1 << 20, 256) == (1 << 20) // 1024 * 256 * 4
+    assert lib.xma_grouped_gemm_workspace_bytes(8, 16384) >= (4 + 2 * (16384 // 128 + 8)) * 4
+
+
+def test_struct_layout_matches_header_field_order():
+    text = open(HEADER).read()
+    body = text[text.index("typedef struct xma_grouped_gemm_args {") : text.index("} xma_grouped_gemm_args;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = re.findall(r"\b(?:const\s+)?(?:void|int32_t|int64_t)\s*\*?\s*([a-z_0-9]+)\s*;", body)
+    assert fields == [f[0] for f in _native.GroupedGemmArgs._fields_]
+
+
+def test_public_surface_mirrors_the_reference_names():
+    for name in ["MoE", "continuous_count", "swiglu", "swiglu_packed", "KernelBackend", "Accelerator", "xma_op",
+                 "CustomOp", "enable_counters", "get_counter_value", "reset_counters", "set_seed"]:
+        assert hasattr(xma, name), name
+    assert [b.value for b in xma.KernelBackend] == ["cuda", "nki", "pallas", "rocm", "torch", "triton"]
+    assert xma.Accelerator.get_kernel_backend() is xma.KernelBackend.rocm
+    for op in ["continuous_count_rocm", "scatter2scatter", "group", "group_bwd_W", "swiglu_forward_rocm",
+               "swiglu_backward_rocm", "route_build_rocm", "topk_softmax_rocm"]:
+        assert hasattr(torch.ops.xma, op), f"xma::{op} is not registered"
+
+
+def test_moe_module_layout_and_state_dict():
+    moe = xma.MoE(num_experts=4, num_experts_per_tok=2, hidden_size=16, intermediate_size=24,
+                  activation_function=xma.swiglu_packed, is_glu=True, add_bias=False, std=0.02)
+    assert moe.c_fc.weight.shape == (4, 48, 16) and moe.c_proj.weight.shape == (4, 16, 24)
+    assert moe.gate.weight.shape == (4, 16) and moe.top_k == 2
+    keys = set(moe.state_dict().keys())
+    assert keys == {"gate.weight", "c_fc.weight", "c_fc.N_array", "c_fc.K_array", "c_proj.weight",
+                    "c_proj.N_array", "c_proj.K_array"}
+    assert moe.c_fc.N_array.tolist() == [48] * 4 and moe.c_fc.K_array.tolist() == [16] * 4
+    assert abs(moe.c_fc.weight.std().item() - 0.02) < 5e-3
+    biased = xma.MoE(2, 1, 8, 8, torch.nn.GELU(), False, True, 0.02)
+    assert biased.c_fc.bias.shape == (2, 8) and torch.all(biased.c_fc.bias == 0)
+
+
+def test_unknown_backends_are_rejected():
+    x = torch.zeros(4, dtype=torch.int32)
+    for backend in (xma.KernelBackend.torch, xma.KernelBackend.triton, xma.KernelBackend.cuda, "rocm"):
+        with pytest.raises(ValueError):
+            xma.continuous_count(x, 8, kernel_backend=backend)
+        with pytest.raises(ValueError):
+            xma.swiglu_packed(torch.zeros(2, 4), kernel_backend=backend)
+    moe = xma.MoE(2, 1, 8, 8, xma.swiglu_packed, True, False, 0.02)
+    with pytest.raises(ValueError):
+        moe(torch.zeros(3, 8), kernel_backend=xma.KernelBackend.torch)
+
+
+def test_cpu_tensors_fail_loudly_instead_of_falling_back():
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        xma.continuous_count(torch.zeros(4, dtype=torch.int32), 8)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        xma.swiglu(torch.zeros(2, 8), torch.zeros(2, 8))
+    assert xma.continuous_count(torch.zeros(5, dtype=torch.int32), 1).tolist() == [5]  # host-only shortcut
+
+
+def test_missing_library_is_an_error(monkeypatch):
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(_native, "_LIB_PATH", "/nonexistent/libxma_hip.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _native.load()
+
+
+def test_counters_and_argument_checks():
+    xma.reset_counters()
+    with xma.enable_counters():
+        with pytest.raises(RuntimeError):
+            xma.swiglu_packed(torch.zeros(2, 4))
+    assert xma.get_counter_value("_SwigluPacked-rocm") == 1
+    with pytest.raises(AssertionError):
+        xma.continuous_count(torch.zeros(2, 2, dtype=torch.int32), 4)  # not 1-D
+    with pytest.raises(AssertionError):
+        xma.continuous_count(torch.zeros(4), 4)  # not an integer tensor
+    with pytest.raises(AssertionError):
+        xma.swiglu(torch.zeros(2, 4), torch.zeros(2, 5))
+    with pytest.raises(AssertionError):
+        xma.swiglu_packed(torch.zeros(2, 5))

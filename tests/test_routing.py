@@ -1,0 +1,131 @@
+"""Router top-k + softmax and the stable counting sort on the GPU: indices, counts, offsets and the
+permutation must be bit-exact against the oracle; routing weights within the float tolerance."""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import flash_model_architectures_amd as xma
+from oracle import torch_oracle as to
+
+from .helpers import TOL, assert_close, assert_same_ints, zipf_bias
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _check_route(ids: torch.Tensor, E: int, index_dtype=torch.int32):
+    r = xma.route_tokens(ids.cuda(), E, index_dtype=index_dtype)
+    o = to.route(ids.flatten().long(), E)
+    assert r.expert_frequency.dtype == torch.uint32 and r.expert_offsets.dtype == torch.int32
+    assert_same_ints(r.expert_frequency, o.expert_frequency, "counts")
+    assert_same_ints(r.expert_offsets, o.expert_offsets, "offsets")
+    assert_same_ints(r.sorted_expert_idxs, o.sorted_expert_idxs, "sorted ids")
+    assert_same_ints(r.sorted_scattered_idxs, o.sorted_scattered_idxs, "permutation")
+    return r
+
+
+@pytest.mark.parametrize("n,E", [(1, 1), (2, 8), (14, 8), (63, 2), (64, 2), (65, 3), (1023, 8), (1024, 8), (1025, 8),
+                                 (4096, 64), (98304, 64), (131072, 128), (5000, 1000), (20000, 16384)])
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
+def test_route_matches_oracle(n, E, dtype):
+    g = torch.Generator().manual_seed(n + E)
+    ids = torch.randint(0, E, (n,), generator=g, dtype=dtype)
+    if E >= 8:
+        ids[ids == 3] = 5  # an empty group in the middle
+    _check_route(ids, E, index_dtype=torch.int64 if dtype == torch.int64 else torch.int32)
+
+
+def test_route_edge_cases():
+    _check_route(torch.zeros(3000, dtype=torch.int64), 8)  # everything on the first expert
+    _check_route(torch.full((3000,), 7, dtype=torch.int32), 8)  # ... on the last
+    _check_route(torch.arange(4096, dtype=torch.int32) % 128, 128)  # perfectly uniform
+    r = xma.route_tokens(torch.empty(0, dtype=torch.int64, device="cuda"), 4)
+    assert r.expert_frequency.tolist() == [0] * 4 and r.expert_offsets.tolist() == [0] * 5
+    _check_route(torch.randint(0, 8, (16, 2)), 8)  # a [tokens, top_k] tensor is flattened row-major
+
+
+def test_route_golden_fixture():
+    z = np.load(os.path.join(GOLDEN, "routing_n64_e8.npz"))
+    r = xma.route_tokens(torch.from_numpy(z["ids"]).cuda(), 8)
+    assert r.expert_frequency.tolist() == z["counts"].tolist()
+    assert r.expert_offsets.tolist() == z["offsets"].tolist()
+    assert r.sorted_scattered_idxs.tolist() == z["perm"].tolist()
+    assert r.sorted_expert_idxs.tolist() == z["sorted_ids"].tolist()
+
+
+def test_route_full_size_invariants():
+    """2^20 ids in [0, 256): exact against the oracle plus the invariants of a stable grouping."""
+
+    torch.manual_seed(0)
+    n, E = 1 << 20, 256
+    ids = torch.randint(0, E, (n,), dtype=torch.int32)
+    r = _check_route(ids, E)
+    perm = r.sorted_scattered_idxs.long()
+    d = ids.cuda()
+    s = d[perm]
+    assert torch.equal(torch.sort(perm).values, torch.arange(n, device="cuda"))
+    assert bool(torch.all(s[1:] >= s[:-1]))
+    same = s[1:] == s[:-1]
+    assert bool(torch.all(perm[1:][same] > perm[:-1][same]))
+
+
+@pytest.mark.parametrize("T,E,k", [(100, 8, 2), (1000, 64, 6), (1000, 128, 8), (64, 8, 1), (33, 300, 4), (7, 600, 8),
+                                   (5, 1000, 3), (3, 8, 8), (50, 2, 2)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_topk_softmax_matches_oracle(T, E, k, dtype):
+    g = torch.Generator().manual_seed(T * 7 + E + k)
+    logits = (torch.randn(T, E, generator=g) * 0.9).to(dtype)  # 16-bit values tie often
+    logits[0, :] = 0.25  # a fully tied row
+    w, idx = xma.topk_softmax(logits.cuda(), k)
+    ow, oidx = to.routing_weights(logits, k)
+    assert idx.dtype == torch.int64 and w.dtype == dtype
+    assert_same_ints(idx, oidx, "selected experts")
+    assert_close(w, ow, TOL[dtype], "routing weights")
+    assert idx[0].tolist() == list(range(k))
+
+
+def test_topk_softmax_golden_and_special_values():
+    z = np.load(os.path.join(GOLDEN, "topk_t12_e16_k4.npz"))
+    w, idx = xma.topk_softmax(torch.from_numpy(z["logits"]).cuda(), 4)
+    assert idx.cpu().tolist() == z["idx"].tolist()
+    assert np.abs(w.cpu().numpy() - z["weights"]).max() < 1e-6
+    special = torch.tensor([[0.0, -0.0, float("-inf"), 1.0], [float("inf"), 1.0, float("inf"), 0.0]])
+    _, idx = xma.topk_softmax(special.cuda(), 2)
+    assert idx.cpu().tolist() == [[3, 0], [0, 2]]  # -0 == +0 ties to the lower index; infs tie too
+    w1, _ = xma.topk_softmax(torch.randn(9, 5).cuda(), 1)
+    assert bool(torch.all(w1 == 1.0))
+
+
+def test_topk_softmax_skewed_full_size():
+    """16384 x 128 bf16 logits with a Zipf(1.2) bias: the skewed-routing workload's router."""
+
+    torch.manual_seed(0)
+    logits = (torch.randn(16384, 128) + zipf_bias(128, 1.2, 2.0)).to(torch.bfloat16)
+    w, idx = xma.topk_softmax(logits.cuda(), 8)
+    ow, oidx = to.routing_weights(logits, 8)
+    assert_same_ints(idx, oidx)
+    assert_close(w, ow, TOL[torch.bfloat16])
+    r = xma.route_tokens(idx, 128)
+    o = to.route(oidx, 128)
+    assert_same_ints(r.sorted_scattered_idxs, o.sorted_scattered_idxs)
+    assert_same_ints(r.expert_frequency, o.expert_frequency)
+    assert int((o.expert_frequency.to(torch.int64) == 0).sum()) >= 1  # ragged and empty groups are present
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_topk_softmax_backward(dtype):
+    g = torch.Generator().manual_seed(5)
+    T, E, k = 257, 64, 6
+    logits = torch.randn(T, E, generator=g).to(dtype)
+    dw = torch.randn(T, k, generator=g).to(dtype)
+    lg = logits.cuda().requires_grad_()
+    w, idx = xma.topk_softmax(lg, k)
+    w.backward(dw.cuda())
+    lo = logits.clone().requires_grad_()
+    ow, _ = to.routing_weights(lo, k)
+    ow.backward(dw)
+    assert_close(lg.grad, lo.grad, TOL[dtype] * (1 if dtype == torch.float32 else 1), "d_logits")
+    assert int((lg.grad != 0).sum(dim=-1).max()) <= k
