@@ -17,16 +17,9 @@
 // tiles (expert, first row), so ragged and empty groups cost nothing; the main kernel renumbers
 // work-groups so that each of the 8 XCDs (private L2 each) owns a contiguous range of tiles, and
 // walks tiles in bands of 4 row tiles x all column tiles to reuse both panels from L2.
-#include "common.h"
+#include "grouped_gemm_common.h"
 
 namespace xma {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
-typedef __attribute__((ext_vector_type(16))) float f32x16_t;
-
-constexpr int kNumXcd = 8;
-constexpr int kBandTiles = 4;  // row tiles per band of the tile walk
 
 // ---- per-dtype tile configuration -----------------------------------------------------------
 template <typename T>
@@ -45,34 +38,6 @@ __device__ __forceinline__ int swizzle_of_row(int row) { return ((row >> 1) ^ (r
 __device__ __forceinline__ int lds_chunk_offset(int row, int chunk) {
     return row * kLdsRowBytes + ((chunk ^ swizzle_of_row(row)) << 4);
 }
-
-// ---- MFMA wrappers: acc(32x32) += X(32 rows x kslice) * Y(32 cols x kslice)^T ----------------------
-template <typename T>
-struct Mma;
-template <>
-struct Mma<bf16_t> {
-    __device__ static __forceinline__ void run(const uint4& x, const uint4& y, f32x16_t& acc) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, x), __builtin_bit_cast(bf16x8_t, y),
-                                                      acc, 0, 0, 0);
-    }
-};
-template <>
-struct Mma<f16_t> {
-    __device__ static __forceinline__ void run(const uint4& x, const uint4& y, f32x16_t& acc) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, x), __builtin_bit_cast(f16x8_t, y),
-                                                     acc, 0, 0, 0);
-    }
-};
-template <>
-struct Mma<float> {
-    // a 16-byte fragment holds 4 reduction steps per lane half; one 32x32x2 MFMA per component
-    __device__ static __forceinline__ void run(const uint4& x, const uint4& y, f32x16_t& acc) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.x), __uint_as_float(y.x), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.y), __uint_as_float(y.y), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.z), __uint_as_float(y.z), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.w), __uint_as_float(y.w), acc, 0, 0, 0);
-    }
-};
 
 // ---- register transposes of a PV x PV block ---------------------------------------------------
 // in[r] = PV consecutive elements of block row r; out[c] = the PV elements of block column c.
@@ -193,66 +158,6 @@ struct TransLoader {
     }
 };
 
-// ---- kernel arguments -----------------------------------------------------------------------------
-struct GemmParams {
-    const void* a;
-    const void* b;
-    void* c;
-    void* aux;
-    const int32_t* offsets;
-    const void* in_index;
-    const void* out_index;
-    const int32_t* tile_expert;  // [row tiles] expert of each row tile (TN/NN)
-    const int32_t* tile_row0;    // [row tiles] first grouped row of each row tile
-    const int32_t* tile_count;   // [1] number of row tiles actually present
-    int64_t lda, ldb, ldc, ld_aux, b_expert_stride, c_expert_stride;
-    int64_t n, k;
-    int32_t num_experts, in_fan_out, idx_is_i64;
-    int32_t row_tiles_max;  // upper bound used for the grid (TN/NN); MT: row tiles per expert
-    int32_t col_tiles;
-};
-
-// routed row p -> source row of the gathered operand (indices are < 2^31, so divide in 32 bits)
-__device__ __forceinline__ int64_t source_row(const GemmParams& P, int64_t p) {
-    return (int64_t)((uint32_t)load_index(P.in_index, P.idx_is_i64, p) / (uint32_t)P.in_fan_out);
-}
-
-// Row-tile list for the row-grouped kinds: expert e owns ceil(count_e / BM) consecutive tiles.
-__global__ __launch_bounds__(1024) void build_row_tiles_kernel(const int32_t* __restrict__ offsets, int E, int BM,
-                                                                int32_t* __restrict__ tile_expert,
-                                                                int32_t* __restrict__ tile_row0,
-                                                                int32_t* __restrict__ tile_count) {
-    __shared__ int32_t part[1024];
-    const int per = (E + 1023) / 1024;
-    const int e0 = threadIdx.x * per;
-    int32_t s = 0;
-    for (int i = 0; i < per; ++i) {
-        const int e = e0 + i;
-        if (e < E) s += (offsets[e + 1] - offsets[e] + BM - 1) / BM;
-    }
-    part[threadIdx.x] = s;
-    __syncthreads();
-    for (int d = 1; d < 1024; d <<= 1) {
-        const int32_t v = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
-        __syncthreads();
-        part[threadIdx.x] += v;
-        __syncthreads();
-    }
-    int32_t t = part[threadIdx.x] - s;
-    for (int i = 0; i < per; ++i) {
-        const int e = e0 + i;
-        if (e < E) {
-            const int32_t begin = offsets[e], end = offsets[e + 1];
-            for (int32_t r = begin; r < end; r += BM) {
-                tile_expert[t] = e;
-                tile_row0[t] = r;
-                ++t;
-            }
-        }
-    }
-    if (threadIdx.x == 1023) tile_count[0] = part[1023];
-}
-
 template <typename T, int KIND, int EPI>
 __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const GemmParams P) {
     using Cfg = TileCfg<T>;
@@ -276,19 +181,9 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
     const int wn0 = (wave % Cfg::WAVES_N) * WN;
 
     // ---- which tile ----
-    // work-groups are dealt round-robin to the XCDs; give each XCD a contiguous range of tiles
-    const int nwg = gridDim.x;  // multiple of kNumXcd
-    const int pid = (blockIdx.x % kNumXcd) * (nwg / kNumXcd) + blockIdx.x / kNumXcd;
     const int row_tiles = KIND == XMA_GEMM_MT ? P.row_tiles_max * P.num_experts : P.tile_count[0];
-    const int col_tiles = P.col_tiles;
-    const int band = pid / (kBandTiles * col_tiles);
-    const int band_first = band * kBandTiles;
-    if (band_first >= row_tiles) return;
-    const int band_rows = row_tiles - band_first < kBandTiles ? row_tiles - band_first : kBandTiles;
-    const int in_band = pid - band * (kBandTiles * col_tiles);
-    const int row_tile = band_first + in_band % band_rows;
-    const int col_tile = in_band / band_rows;
-    if (col_tile >= col_tiles) return;
+    int row_tile, col_tile;
+    if (!locate_tile(row_tiles, P.col_tiles, row_tile, col_tile)) return;
 
     const T* A = reinterpret_cast<const T*>(P.a);
     const T* B = reinterpret_cast<const T*>(P.b);
@@ -559,13 +454,50 @@ constexpr int lds_bytes() {
     return stages > ctile ? stages : ctile;
 }
 
-static int64_t max_row_tiles(int64_t rows, int E, int BM) { return rows / BM + E; }
-
 template <typename T, int KIND, int EPI>
 static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
     using Cfg = TileCfg<T>;
     constexpr int PV = Elem<T>::kPerVec;
     GemmParams P;
+    fill_params(a, P);
+
+    int64_t grid;
+    if (KIND == XMA_GEMM_MT) {
+        P.row_tiles_max = (int32_t)ceil_div(a.n, Cfg::BM);
+        P.col_tiles = (int32_t)ceil_div(a.k, Cfg::BN);
+        grid = grid_for_tiles((int64_t)P.row_tiles_max * a.num_experts, P.col_tiles);
+    } else {
+        const int64_t rt = max_row_tiles(a.rows, a.num_experts, Cfg::BM);
+        int32_t* ws = reinterpret_cast<int32_t*>(a.workspace);
+        P.tile_count = ws;
+        P.tile_expert = ws + 4;
+        P.tile_row0 = ws + 4 + rt;
+        P.row_tiles_max = (int32_t)rt;
+        const int bn_out = EPI == XMA_EPI_SWIGLU ? Cfg::BN / 2 : Cfg::BN;
+        const int64_t n_out = EPI == XMA_EPI_SWIGLU ? a.n / 2 : a.n;
+        P.col_tiles = (int32_t)ceil_div(n_out, bn_out);
+        grid = grid_for_tiles(rt, P.col_tiles);
+        hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(1024), 0, stream, a.expert_offsets, a.num_experts,
+                           Cfg::BM, ws + 4, ws + 4 + rt, ws);
+    }
+    XMA_REQUIRE(grid < ((int64_t)1 << 31), "xma_grouped_gemm: %lld tiles exceed the grid limit", (long long)grid);
+    (void)PV;
+    auto kernel = grouped_gemm_kernel<T, KIND, EPI>;
+    static bool attr_set = false;  // per instantiation
+    if (!attr_set) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<T>());
+        if (err != hipSuccess) {
+            set_error("xma_grouped_gemm: cannot reserve %d bytes of LDS: %s", lds_bytes<T>(), hipGetErrorString(err));
+            return 2;
+        }
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(Cfg::THREADS), lds_bytes<T>(), stream, P);
+    return check_launch("xma_grouped_gemm");
+}
+
+void fill_params(const xma_grouped_gemm_args& a, GemmParams& P) {
     P.a = a.a;
     P.b = a.b;
     P.c = a.c;
@@ -587,43 +519,8 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
     P.tile_expert = nullptr;
     P.tile_row0 = nullptr;
     P.tile_count = nullptr;
-
-    int64_t tiles;
-    if (KIND == XMA_GEMM_MT) {
-        P.row_tiles_max = (int32_t)ceil_div(a.n, Cfg::BM);
-        P.col_tiles = (int32_t)ceil_div(a.k, Cfg::BN);
-        tiles = ceil_div((int64_t)P.row_tiles_max * a.num_experts, kBandTiles) * kBandTiles * P.col_tiles;
-    } else {
-        const int64_t rt = max_row_tiles(a.rows, a.num_experts, Cfg::BM);
-        int32_t* ws = reinterpret_cast<int32_t*>(a.workspace);
-        P.tile_count = ws;
-        P.tile_expert = ws + 4;
-        P.tile_row0 = ws + 4 + rt;
-        P.row_tiles_max = (int32_t)rt;
-        const int bn_out = EPI == XMA_EPI_SWIGLU ? Cfg::BN / 2 : Cfg::BN;
-        const int64_t n_out = EPI == XMA_EPI_SWIGLU ? a.n / 2 : a.n;
-        P.col_tiles = (int32_t)ceil_div(n_out, bn_out);
-        // whole bands of kBandTiles row tiles, so that every present row tile has a work-group
-        tiles = ceil_div(rt, kBandTiles) * kBandTiles * P.col_tiles;
-        hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(1024), 0, stream, a.expert_offsets, a.num_experts,
-                           Cfg::BM, ws + 4, ws + 4 + rt, ws);
-    }
-    const int64_t grid = ceil_div(tiles, kNumXcd) * kNumXcd;
-    XMA_REQUIRE(grid < ((int64_t)1 << 31), "xma_grouped_gemm: %lld tiles exceed the grid limit", (long long)grid);
-    (void)PV;
-    auto kernel = grouped_gemm_kernel<T, KIND, EPI>;
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<T>());
-        if (err != hipSuccess) {
-            set_error("xma_grouped_gemm: cannot reserve %d bytes of LDS: %s", lds_bytes<T>(), hipGetErrorString(err));
-            return 2;
-        }
-        attr_set = true;
-    }
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(Cfg::THREADS), lds_bytes<T>(), stream, P);
-    return check_launch("xma_grouped_gemm");
+    P.row_tiles_max = 0;
+    P.col_tiles = 0;
 }
 
 template <typename T>
@@ -704,6 +601,7 @@ int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
     }
     XMA_REQUIRE(a.a && a.b && a.c, "xma_grouped_gemm: null operand");
     hipStream_t stream = (hipStream_t)stream_;
+    if (dma_gemm_supports(a)) return launch_dma_gemm(a, stream);
     switch (a.dtype) {
         case XMA_F32:
             return dispatch_kind<float>(a, stream);

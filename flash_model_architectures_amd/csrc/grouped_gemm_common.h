@@ -1,0 +1,142 @@
+// Pieces shared by the grouped-GEMM kernels: kernel arguments, the row-tile list that maps
+// work-groups to (expert, rows) without host synchronisation, and the XCD-aware tile walk.
+#pragma once
+
+#include "common.h"
+
+namespace xma {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // 16 bytes moved as ONE vector access
+
+constexpr int kNumXcd = 8;     // accelerator complex dies, each with a private L2
+constexpr int kBandTiles = 4;  // row tiles per band of the tile walk
+
+// ---- kernel arguments -----------------------------------------------------------------------------
+struct GemmParams {
+    const void* a;
+    const void* b;
+    void* c;
+    void* aux;
+    const int32_t* offsets;
+    const void* in_index;
+    const void* out_index;
+    const int32_t* tile_expert;  // [row tiles] expert of each row tile (TN/NN)
+    const int32_t* tile_row0;    // [row tiles] first grouped row of each row tile
+    const int32_t* tile_count;   // [1] number of row tiles actually present
+    int64_t lda, ldb, ldc, ld_aux, b_expert_stride, c_expert_stride;
+    int64_t n, k;
+    int32_t num_experts, in_fan_out, idx_is_i64;
+    int32_t row_tiles_max;  // upper bound used for the grid (TN/NN); MT: row tiles per expert
+    int32_t col_tiles;
+};
+
+// routed row p -> source row of the gathered operand (indices are < 2^31, so divide in 32 bits)
+__device__ __forceinline__ int64_t source_row(const GemmParams& P, int64_t p) {
+    return (int64_t)((uint32_t)load_index(P.in_index, P.idx_is_i64, p) / (uint32_t)P.in_fan_out);
+}
+
+// Row-tile list for the row-grouped kinds: expert e owns ceil(count_e / BM) consecutive tiles.
+static __global__ __launch_bounds__(1024) void build_row_tiles_kernel(const int32_t* __restrict__ offsets, int E, int BM,
+                                                                int32_t* __restrict__ tile_expert,
+                                                                int32_t* __restrict__ tile_row0,
+                                                                int32_t* __restrict__ tile_count) {
+    __shared__ int32_t part[1024];
+    const int per = (E + 1023) / 1024;
+    const int e0 = threadIdx.x * per;
+    int32_t s = 0;
+    for (int i = 0; i < per; ++i) {
+        const int e = e0 + i;
+        if (e < E) s += (offsets[e + 1] - offsets[e] + BM - 1) / BM;
+    }
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        const int32_t v = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+        __syncthreads();
+        part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    int32_t t = part[threadIdx.x] - s;
+    for (int i = 0; i < per; ++i) {
+        const int e = e0 + i;
+        if (e < E) {
+            const int32_t begin = offsets[e], end = offsets[e + 1];
+            for (int32_t r = begin; r < end; r += BM) {
+                tile_expert[t] = e;
+                tile_row0[t] = r;
+                ++t;
+            }
+        }
+    }
+    if (threadIdx.x == 1023) tile_count[0] = part[1023];
+}
+
+
+// Work-group -> (row tile, column tile).  Work-groups are dealt round-robin to the XCDs, so the
+// block index is first renumbered to give every XCD a contiguous range of tiles; tiles are then
+// walked in bands of kBandTiles row tiles x all column tiles, row tile fastest, so that work-groups
+// running at the same time share A row panels and B column panels in their XCD's L2.
+// Returns false when this work-group has no tile.
+__device__ __forceinline__ bool locate_tile(int row_tiles, int col_tiles, int& row_tile, int& col_tile) {
+    const int nwg = gridDim.x;  // a multiple of kNumXcd
+    const int pid = (blockIdx.x % kNumXcd) * (nwg / kNumXcd) + blockIdx.x / kNumXcd;
+    const int band = pid / (kBandTiles * col_tiles);
+    const int band_first = band * kBandTiles;
+    if (band_first >= row_tiles) return false;
+    const int band_rows = row_tiles - band_first < kBandTiles ? row_tiles - band_first : kBandTiles;
+    const int in_band = pid - band * (kBandTiles * col_tiles);
+    row_tile = band_first + in_band % band_rows;
+    col_tile = in_band / band_rows;
+    return col_tile < col_tiles;
+}
+
+// number of work-groups that covers `row_tiles` x `col_tiles` under locate_tile()
+inline int64_t grid_for_tiles(int64_t row_tiles, int64_t col_tiles) {
+    const int64_t tiles = ceil_div(row_tiles, kBandTiles) * kBandTiles * col_tiles;
+    return ceil_div(tiles, kNumXcd) * kNumXcd;
+}
+
+inline int64_t max_row_tiles(int64_t rows, int E, int BM) { return rows / BM + E; }
+
+// The MFMA instruction the 16-bit kernels are built on: acc(32x32) += X(32 x 16) * Y(32 x 16)^T,
+// lane l supplies row l%32 and the 8 reduction elements 8*(l/32)..8*(l/32)+7 of both operands.
+template <typename T>
+struct Mma;
+template <>
+struct Mma<bf16_t> {
+    template <typename V>
+    __device__ static __forceinline__ void run(const V& x, const V& y, f32x16_t& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, x), __builtin_bit_cast(bf16x8_t, y),
+                                                      acc, 0, 0, 0);
+    }
+};
+template <>
+struct Mma<f16_t> {
+    template <typename V>
+    __device__ static __forceinline__ void run(const V& x, const V& y, f32x16_t& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, x), __builtin_bit_cast(f16x8_t, y),
+                                                     acc, 0, 0, 0);
+    }
+};
+template <>
+struct Mma<float> {
+    // a 16-byte fragment holds 4 reduction steps per lane half; one 32x32x2 MFMA per component
+    __device__ static __forceinline__ void run(const uint4& x, const uint4& y, f32x16_t& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.x), __uint_as_float(y.x), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.y), __uint_as_float(y.y), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.z), __uint_as_float(y.z), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(x.w), __uint_as_float(y.w), acc, 0, 0, 0);
+    }
+};
+
+// Fills the fields of GemmParams that do not depend on the tile shape.
+void fill_params(const xma_grouped_gemm_args& a, GemmParams& P);
+
+// The LDS-DMA pipelined kernel for 16-bit element types (grouped_gemm_dma.hip).
+bool dma_gemm_supports(const xma_grouped_gemm_args& a);
+int launch_dma_gemm(const xma_grouped_gemm_args& a, hipStream_t stream);
+
+}  // namespace xma
