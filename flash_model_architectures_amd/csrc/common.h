@@ -125,6 +125,10 @@ struct Elem<f16_t> {
 // sigmoid in fp32 with an accurate exponential
 __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
 
+// sigmoid from the hardware exp2 and reciprocal (a few ulp in fp32): for results that are rounded to a
+// 16-bit type anyway
+__device__ __forceinline__ float sigmoid_fast(float x) { return __frcp_rn(1.0f + __expf(-x)); }
+
 // ---- wave64 primitives ------------------------------------------------------------------------
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (kWaveSize - 1)); }
 

@@ -1,16 +1,20 @@
 // Ragged (per-expert) GEMM for 16-bit element types on gfx950, built around the LDS-DMA load path
-// (global_load_lds_dwordx4): tiles travel HBM -> LDS without passing through registers, four
-// 32-deep stages are kept in LDS so that three stages of loads are always in flight while the
-// fourth is multiplied, and operands whose reduction index is strided in HBM are fetched in their
-// HBM layout and transposed by the LDS read itself (ds_read_b64_tr_b16).
+// (global_load_lds_dwordx4): tiles travel L2 -> LDS without passing through registers, several
+// stages are kept in LDS so that loads stay in flight while a stage is multiplied, and operands whose
+// reduction index is strided in HBM are fetched in their HBM layout and transposed by the LDS read
+// itself (ds_read_b64_tr_b16).
 //
 // Tile 256 x 256 per work-group, 8 waves as 2 x 4, each wave 128 x 64 (4 x 2 MFMA 32x32x16 tiles).
 //
-// LDS layouts (one 32 KiB array per stage: 16 KiB per operand):
-//   K-contiguous operand (A in TN/NN, W in TN): [256 tile rows][32 k], 64 bytes per row; the four
-//     16-byte chunks of row r sit at chunk ^ ((r >> 2) & 3), so that the 16 rows a quarter-wave reads
-//     in one ds_read_b128 cover all 64 banks.
-//   K-strided operand (W in NN, both operands in MT): [32 k][256 tile rows], 512 bytes per k row; chunk c
+// LDS is a pool of four 32 KiB slabs; the pipeline policy Pipe32x4 keeps four stages of 32 reduction
+// elements in them, one slab each (A tile | B tile), with three stages of loads in flight.  (A variant
+// with 64-deep blocks rotating through five slabs, so that every DMA instruction asks for whole 128-byte
+// lines, measured the same or slower on the layer's shapes and was dropped.)
+// Tile layouts inside a slab:
+//   K-contiguous operand (A in TN/NN, W in TN): [256 tile rows][BK k]; the 16-byte chunks of a row are
+//     XOR-swizzled by the row number so that the 16 rows a quarter-wave reads in one ds_read_b128 cover all
+//     64 banks.
+//   K-strided operand (W in NN, both operands in MT): [BK k][256 tile rows], 512 bytes per k row; chunk c
 //     of k row r sits at c ^ ((r & 3) << 2), so that the four k rows one transposing read touches fall
 //     into different bank groups.
 // A DMA load writes lane l's 16 bytes at (wave-uniform LDS base) + 16*l, so the swizzles are applied
@@ -21,32 +25,31 @@
 namespace xma {
 namespace dma {
 
-constexpr int BM = 256, BN = 256, BK = 32, NS = 4, THREADS = 512;
+constexpr int BM = 256, BN = 256, THREADS = 512;
 constexpr int WAVES_N = 4, WM = 128, WN = 64, MI = WM / 32, NI = WN / 32;
-constexpr int OPERAND_BYTES = BM * BK * 2;  // 16 KiB, same for both layouts and both operands
-constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;
-constexpr int LOADS_PER_STAGE = 4;          // DMA instructions per wave per stage (2 per operand)
+constexpr int SLAB_BYTES = 32768;
 static_assert(BM == BN, "both operands use the same tile height");
 
-__shared__ __attribute__((aligned(1024))) char stage0[STAGE_BYTES];
-__shared__ __attribute__((aligned(1024))) char stage1[STAGE_BYTES];
-__shared__ __attribute__((aligned(1024))) char stage2[STAGE_BYTES];
-__shared__ __attribute__((aligned(1024))) char stage3[STAGE_BYTES];
+__shared__ __attribute__((aligned(1024))) char slab0[SLAB_BYTES];
+__shared__ __attribute__((aligned(1024))) char slab1[SLAB_BYTES];
+__shared__ __attribute__((aligned(1024))) char slab2[SLAB_BYTES];
+__shared__ __attribute__((aligned(1024))) char slab3[SLAB_BYTES];
 
-// The stages are distinct arrays on purpose: the compiler can then prove that a fragment read of
-// one stage does not alias the DMA writes still in flight to the others, and does not drain them.
-template <int S>
-__device__ __forceinline__ char* stage_ptr() {
-    static_assert(S >= 0 && S < NS, "stage index");
-    if constexpr (S == 0) return stage0;
-    if constexpr (S == 1) return stage1;
-    if constexpr (S == 2) return stage2;
-    return stage3;
+// The slabs are distinct arrays on purpose: the compiler can then prove that a fragment read of
+// one slab does not alias the DMA writes still in flight to the others, and does not drain them.
+template <int I>
+__device__ __forceinline__ char* slab() {
+    static_assert(I >= 0 && I < 4, "slab index");
+    if constexpr (I == 0) return slab0;
+    if constexpr (I == 1) return slab1;
+    if constexpr (I == 2) return slab2;
+    return slab3;
 }
 
 __device__ __attribute__((aligned(16))) uint32_t g_zero_page[4];  // zero-initialised
 
 typedef __attribute__((ext_vector_type(4))) short short4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 #define XMA_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define XMA_LDS_S4(p) ((__attribute__((address_space(3))) short4_t*)(p))
 
@@ -67,142 +70,194 @@ __device__ __forceinline__ void block_barrier() {
     compiler_fence();
 }
 
-// Per-thread state of one operand's DMA loads: two loads per stage.
-template <typename T>
-struct OperandLoads {
-    const T* ptr[2];    // HBM address of this lane's chunk in stage 0 (or the zero page)
-    int64_t step;       // elements to advance per stage
-    int32_t red[2];     // reduction index covered by the lane in stage 0 (chunk start or k row)
-    bool valid[2];      // false: always the zero page (row / column outside the operand)
-    int lds_off[2];     // byte offset of the wave's 1 KiB destination inside the operand's LDS tile
-};
-
-// K-contiguous layout: wave w fills tile rows [16w, 16w+16) and [128 + 16w, ...): lane l -> row + l/4,
-// physical chunk l%4.  row_fn(tile row) returns the HBM row base or nullptr.
-template <typename T, typename RowFn>
-__device__ __forceinline__ void setup_kcontig(OperandLoads<T>& L, int wave, int lane, RowFn row_fn) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int row = i * 128 + wave * 16 + (lane >> 2);
-        const int chunk = (lane & 3) ^ ((row >> 2) & 3);  // logical chunk stored at physical position lane&3
-        const T* base = row_fn(row);
-        L.valid[i] = base != nullptr;
-        L.ptr[i] = L.valid[i] ? base + chunk * 8 : reinterpret_cast<const T*>(g_zero_page);
-        L.red[i] = chunk * 8;
-        L.lds_off[i] = (i * 128 + wave * 16) * (BK * 2);
-    }
-    L.step = BK;
-}
-
-// K-strided layout: wave w fills k rows {2w, 2w+1} and {16 + 2w, 16 + 2w + 1}: lane l -> k row + l/32,
-// physical chunk l%32.  `base` points at (reduction row 0, first tile column); `cols_left` = number of
-// valid columns from there; ld = row stride.
-template <typename T>
-__device__ __forceinline__ void setup_kstrided(OperandLoads<T>& L, int wave, int lane, const T* base, int64_t ld,
-                                               int64_t cols_left) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int krow = i * 16 + wave * 2 + (lane >> 5);
-        const int chunk = (lane & 31) ^ ((krow & 3) << 2);
-        L.valid[i] = chunk * 8 < cols_left;
-        L.ptr[i] = L.valid[i] ? base + (int64_t)krow * ld + chunk * 8 : reinterpret_cast<const T*>(g_zero_page);
-        L.red[i] = krow;
-        L.lds_off[i] = (i * 16 + wave * 2) * (BN * 2);
-    }
-    L.step = (int64_t)BK * ld;
-}
-
-// Issue this wave's two loads of one operand for the stage starting at reduction index k0.
-template <typename T>
-__device__ __forceinline__ void issue_operand(const OperandLoads<T>& L, char* lds_stage, int operand_off, int64_t stage,
-                                              int64_t k0, int64_t red_len) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const bool ok = L.valid[i] && (k0 + L.red[i] < red_len);
-        const T* src = ok ? L.ptr[i] + stage * L.step : reinterpret_cast<const T*>(g_zero_page);
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(src),
-                                         XMA_LDS(lds_stage + (operand_off + L.lds_off[i])), 16, 0, 0);
-    }
-}
-
-// LDS accesses below add ONE integer byte offset to the stage array, and the offset is passed through
-// opaque() so that the optimiser cannot split it into a chain of partial sums: the compiler attaches the
-// "this access belongs to stage array X" information it needs to keep DMA loads to the other arrays in
-// flight only to accesses whose address is a short derivation from the array.
+// LDS accesses add ONE integer byte offset to a slab, and the variable part of the offset is passed
+// through opaque() so that the optimiser cannot split it into a chain of partial sums: the compiler
+// attaches the "this access belongs to slab X" information it needs to keep DMA loads to the other
+// slabs in flight only to accesses whose address is a short derivation from the array.
 __device__ __forceinline__ int opaque(int v) {
     asm("" : "+v"(v));
     return v;
 }
 
-// Fragment of a K-contiguous tile: row `row`, reduction elements kk*16 + 8*half .. +7.
-__device__ __forceinline__ int kcontig_offset(int row, int kk, int half) {
-    const int chunk = (2 * kk + half) ^ ((row >> 2) & 3);
-    return row * (BK * 2) + (chunk << 4);
-}
+// ---- tile geometry for a stage depth of BK reduction elements ---------------------------------------
+template <int BK>
+struct Geometry {
+    static constexpr int CPR = BK / 8;            // 16-byte chunks per K-contiguous row
+    static constexpr int ROW_BYTES = BK * 2;
+    static constexpr int ROWS_PER_LOAD = 64 / CPR;  // tile rows one DMA instruction covers
+    static constexpr int LOADS = BK / 16;         // DMA instructions per wave, operand and stage
+    static constexpr int TILE_BYTES = BM * BK * 2;
+    static_assert(BK == 32 || BK == 64, "stage depth");
 
-// Same fragment out of a K-strided tile, transposed by the LDS read.  Within each 16-lane group the
-// instruction hands lane i the i-th 16-bit element of four 16-element rows, where row j is assembled from
-// the 8-byte pieces addressed by lanes 4j..4j+3.  So lane i addresses (k row 4*j' + i/4, columns 4*(i%4)..+3)
-// and receives four consecutive k of column i; a second read four k rows further down completes the
-// eight reduction elements of the MFMA operand.
-__device__ __forceinline__ int kstrided_offset(int col0, int kk, int lane) {
-    const int i = lane & 15, group = lane >> 4;
-    const int col = col0 + 16 * (group & 1) + 4 * (i & 3);
-    const int krow0 = kk * 16 + 8 * (group >> 1) + (i >> 2);
-    const int chunk = (col >> 3) ^ ((krow0 & 3) << 2);  // (krow0 + 4) & 3 == krow0 & 3
-    return krow0 * (BN * 2) + (chunk << 4) + ((col & 4) << 1);
-}
+    __device__ static __forceinline__ int swizzle(int row) { return BK == 32 ? (row >> 2) & 3 : (row >> 1) & 7; }
 
-typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+    // K-contiguous tile: byte offset of the fragment (row, reduction elements kk*16 + 8*half .. +7)
+    __device__ static __forceinline__ int kcontig_offset(int row, int kk, int half) {
+        return row * ROW_BYTES + (((2 * kk + half) ^ swizzle(row)) << 4);
+    }
+    // K-strided tile: byte offset of the first of the two transposing reads of the fragment
+    // (tile rows col0..col0+31, reduction elements kk*16 .. +15).  Within each 16-lane group the
+    // instruction hands lane i the i-th 16-bit element of four 16-element rows, where row j is assembled
+    // from the 8-byte pieces addressed by lanes 4j..4j+3.  So lane i addresses (k row i/4, columns
+    // 4*(i%4)..+3) and receives four consecutive k of column i; a second read four k rows further down
+    // completes the eight reduction elements of the MFMA operand.
+    __device__ static __forceinline__ int kstrided_offset(int col0, int kk, int lane) {
+        const int i = lane & 15, group = lane >> 4;
+        const int col = col0 + 16 * (group & 1) + 4 * (i & 3);
+        const int krow0 = kk * 16 + 8 * (group >> 1) + (i >> 2);
+        const int chunk = (col >> 3) ^ ((krow0 & 3) << 2);  // (krow0 + 4) & 3 == krow0 & 3
+        return krow0 * (BN * 2) + (chunk << 4) + ((col & 4) << 1);
+    }
+};
 
 template <bool STRIDED>
-__device__ __forceinline__ u32x4_t read_fragment(const char* stage, int offset) {
+__device__ __forceinline__ u32x4_t read_fragment(const char* slab_base, int offset) {
     if constexpr (STRIDED) {
-        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(XMA_LDS_S4(stage + offset));
-        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(XMA_LDS_S4(stage + (offset + 4 * (BN * 2))));
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(XMA_LDS_S4(slab_base + offset));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(XMA_LDS_S4(slab_base + (offset + 4 * (BN * 2))));
         const u32x2_t a = __builtin_bit_cast(u32x2_t, lo), b = __builtin_bit_cast(u32x2_t, hi);
         return u32x4_t{a.x, a.y, b.x, b.y};
     } else {
-        return *reinterpret_cast<const u32x4_t*>(stage + offset);
+        return *reinterpret_cast<const u32x4_t*>(slab_base + offset);
     }
 }
 
-template <typename T, int KIND, int EPI>
+// ---- per-thread DMA plan of one operand ---------------------------------------------------------------
+template <typename T, int BK>
+struct OperandLoads {
+    static constexpr int LOADS = Geometry<BK>::LOADS;
+    const T* ptr[LOADS];  // HBM address of this lane's chunk in stage 0 (or the zero page)
+    int64_t step;         // elements to advance per stage
+    int32_t red[LOADS];   // reduction index covered by the lane in stage 0 (chunk start or k row)
+    bool valid[LOADS];    // false: always the zero page (row / column outside the operand)
+    int lds_off[LOADS];   // byte offset of the wave's 1 KiB destination inside the operand's LDS tile
+
+    // K-contiguous layout: DMA instruction i of wave w fills tile rows [R*(8i + w), +R), R = ROWS_PER_LOAD:
+    // lane l -> row + l/CPR, physical chunk l%CPR.  row_fn(tile row) returns the HBM row base or nullptr.
+    template <typename RowFn>
+    __device__ __forceinline__ void setup_kcontig(int wave, int lane, RowFn row_fn) {
+        using G = Geometry<BK>;
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int row0 = (i * 8 + wave) * G::ROWS_PER_LOAD;
+            const int row = row0 + lane / G::CPR;
+            const int chunk = (lane % G::CPR) ^ G::swizzle(row);  // logical chunk stored at physical position
+            const T* base = row_fn(row);
+            valid[i] = base != nullptr;
+            ptr[i] = valid[i] ? base + chunk * 8 : reinterpret_cast<const T*>(g_zero_page);
+            red[i] = chunk * 8;
+            lds_off[i] = row0 * G::ROW_BYTES;
+        }
+        step = BK;
+    }
+
+    // K-strided layout: DMA instruction i of wave w fills k rows {2*(8i + w), +1}: lane l -> k row + l/32,
+    // physical chunk l%32.  `base` points at (reduction row 0, first tile column); `cols_left` = number of
+    // valid columns from there; ld = row stride.
+    __device__ __forceinline__ void setup_kstrided(int wave, int lane, const T* base, int64_t ld, int64_t cols_left) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int krow0 = (i * 8 + wave) * 2;
+            const int krow = krow0 + (lane >> 5);
+            const int chunk = (lane & 31) ^ ((krow & 3) << 2);
+            valid[i] = chunk * 8 < cols_left;
+            ptr[i] = valid[i] ? base + (int64_t)krow * ld + chunk * 8 : reinterpret_cast<const T*>(g_zero_page);
+            red[i] = krow;
+            lds_off[i] = krow0 * (BN * 2);
+        }
+        step = (int64_t)BK * ld;
+    }
+
+    // Issue this wave's loads for the stage `stage` into the tile at slab_base + tile_off.
+    __device__ __forceinline__ void issue(char* slab_base, int tile_off, int64_t stage, int64_t red_len) const {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const bool ok = valid[i] && (stage * BK + red[i] < red_len);
+            const T* src = ok ? ptr[i] + stage * step : reinterpret_cast<const T*>(g_zero_page);
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(src),
+                                             XMA_LDS(slab_base + (tile_off + lds_off[i])), 16, 0, 0);
+        }
+    }
+};
+
+// ---- pipeline policies --------------------------------------------------------------------------------------
+// A policy names, for every position P of its unrolled cycle, the slab and offset of the A and B tiles
+// that step P multiplies, what the step loads, and how many younger DMA instructions may stay in flight
+// when the step starts.
+struct Pipe32x4 {
+    static constexpr int BK = 32, CYCLE = 4;
+    static constexpr int WAIT = 2 * 2 * Geometry<BK>::LOADS;  // two younger stages, two operands each
+    template <int P> struct At {
+        static constexpr int A_SLAB = P, A_OFF = 0, B_SLAB = P, B_OFF = Geometry<BK>::TILE_BYTES;
+    };
+    template <typename K> __device__ static __forceinline__ void prologue(K& k) {
+        k.template issue_a<0>(0); k.template issue_b<0>(0);
+        k.template issue_a<1>(1); k.template issue_b<1>(1);
+        k.template issue_a<2>(2); k.template issue_b<2>(2);
+    }
+    // step s refills the slab that step s-1 released with stage s+3
+    template <int P, typename K> __device__ static __forceinline__ void refill(K& k, int64_t s) {
+        k.template issue_a<(P + 3) % CYCLE>(s + 3);
+        k.template issue_b<(P + 3) % CYCLE>(s + 3);
+    }
+};
+
+template <typename T, int KIND, int EPI, typename Pipe>
 struct Kernel {
+    static constexpr int BK = Pipe::BK;
+    using G = Geometry<BK>;
     static constexpr bool A_STRIDED = KIND == XMA_GEMM_MT;
     static constexpr bool B_STRIDED = KIND != XMA_GEMM_TN;
     static constexpr int BN_OUT = EPI == XMA_EPI_SWIGLU ? BN / 2 : BN;
 
-    OperandLoads<T> la, lb;
+    OperandLoads<T, BK> la, lb;
     int64_t red_len;
     int wave, lane;
+    int a_off[4], b_off[4];  // variable parts of the fragment offsets (see fragment_offsets)
 
-    template <int S>
-    __device__ __forceinline__ void issue(int64_t stage) {
-        issue_operand(la, stage_ptr<S>(), 0, stage, stage * BK, red_len);
-        issue_operand(lb, stage_ptr<S>(), OPERAND_BYTES, stage, stage * BK, red_len);
+    template <int P> __device__ __forceinline__ void issue_a(int64_t stage) {
+        la.issue(slab<Pipe::template At<P>::A_SLAB>(), Pipe::template At<P>::A_OFF, stage, red_len);
+    }
+    template <int P> __device__ __forceinline__ void issue_b(int64_t stage) {
+        lb.issue(slab<Pipe::template At<P>::B_SLAB>(), Pipe::template At<P>::B_OFF, stage, red_len);
     }
 
-    template <int S>
+    // Byte offsets of this lane's fragments inside an operand tile.  Only the part that is not a
+    // compile-time constant goes through opaque(): for the K-contiguous layout the tile-row block adds a
+    // constant (32 rows, same swizzle), for the K-strided layout the k16 step does (16 k rows = 8 KiB).
+    template <bool STRIDED, int BLOCKS>
+    __device__ __forceinline__ void fragment_offsets(int row0, int (&var)[4]) const {
+        if constexpr (STRIDED) {
+#pragma unroll
+            for (int b = 0; b < BLOCKS; ++b) var[b] = opaque(G::kstrided_offset(row0 + b * 32, 0, lane));
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < BK / 16; ++kk) var[kk] = opaque(G::kcontig_offset(row0 + (lane & 31), kk, lane >> 5));
+        }
+    }
+    template <bool STRIDED>
+    __device__ static __forceinline__ int fragment_offset(const int (&var)[4], int block, int kk) {
+        return STRIDED ? var[block] + kk * (16 * BN * 2) : var[kk] + block * (32 * G::ROW_BYTES);
+    }
+    __device__ __forceinline__ void init_fragments() {
+        fragment_offsets<A_STRIDED, MI>((wave / WAVES_N) * WM, a_off);
+        fragment_offsets<B_STRIDED, NI>((wave % WAVES_N) * WN, b_off);
+    }
+
+    template <int P>
     __device__ __forceinline__ void compute(f32x16_t (&acc)[MI][NI]) {
-        const char* stage = stage_ptr<S>();
-        const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
-        const int frow = lane & 31, half = lane >> 5;
+        using At = typename Pipe::template At<P>;
+        const char* ta = slab<At::A_SLAB>();
+        const char* tb = slab<At::B_SLAB>();
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
             u32x4_t af[MI], bf[NI];
 #pragma unroll
-            for (int mi = 0; mi < MI; ++mi) {
-                const int off = A_STRIDED ? kstrided_offset(wm0 + mi * 32, kk, lane)
-                                          : kcontig_offset(wm0 + mi * 32 + frow, kk, half);
-                af[mi] = read_fragment<A_STRIDED>(stage, opaque(off));
-            }
+            for (int mi = 0; mi < MI; ++mi)
+                af[mi] = read_fragment<A_STRIDED>(ta, At::A_OFF + fragment_offset<A_STRIDED>(a_off, mi, kk));
 #pragma unroll
-            for (int ni = 0; ni < NI; ++ni) {
-                const int off = B_STRIDED ? kstrided_offset(wn0 + ni * 32, kk, lane)
-                                          : kcontig_offset(wn0 + ni * 32 + frow, kk, half);
-                bf[ni] = read_fragment<B_STRIDED>(stage, opaque(OPERAND_BYTES + off));
-            }
+            for (int ni = 0; ni < NI; ++ni)
+                bf[ni] = read_fragment<B_STRIDED>(tb, At::B_OFF + fragment_offset<B_STRIDED>(b_off, ni, kk));
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -210,23 +265,52 @@ struct Kernel {
         }
     }
 
-    // One pipeline step on stage s (S = s % NS): wait until at most the two younger stages are in
-    // flight, meet the other waves (stage s has landed for everybody and the buffer of stage s-1 is no longer
-    // read), refill that buffer with stage s+3, multiply.  The step is branch-free: stages past the end of
-    // the reduction fetch the zero page, which keeps the count of loads in flight the same at every step and
-    // lets the compiler see that the loop needs no other wait on vector memory.
-    template <int S>
+    // One pipeline step at cycle position P on stage s: wait until only the younger loads named by the
+    // policy are in flight, meet the other waves (stage s has landed for everybody and the slabs of stage
+    // s-1 are no longer read), refill the released slabs, multiply.  A step is branch-free: stages past the
+    // end of the reduction fetch the zero page, which keeps the count of loads in flight the same at every
+    // step and lets the compiler see that the loop needs no other wait on vector memory.
+    template <int P>
     __device__ __forceinline__ void step(int64_t s, f32x16_t (&acc)[MI][NI]) {
-        wait_vmcnt<2 * LOADS_PER_STAGE>();
+        wait_vmcnt<Pipe::WAIT>();
         block_barrier();
-        issue<(S + NS - 1) % NS>(s + NS - 1);
-        compute<S>(acc);
+        Pipe::template refill<P>(*this, s);
+        compute<P>(acc);
+    }
+
+    template <int P>
+    __device__ __forceinline__ void steps_from(int64_t s, int64_t count, f32x16_t (&acc)[MI][NI]) {
+        if constexpr (P < Pipe::CYCLE) {
+            if (P < count) {
+                step<P>(s + P, acc);
+                steps_from<P + 1>(s, count, acc);
+            }
+        }
+    }
+    template <int P>
+    __device__ __forceinline__ void full_cycle(int64_t s, f32x16_t (&acc)[MI][NI]) {
+        if constexpr (P < Pipe::CYCLE) {
+            step<P>(s + P, acc);
+            full_cycle<P + 1>(s, acc);
+        }
+    }
+
+    __device__ __forceinline__ void run(f32x16_t (&acc)[MI][NI]) {
+        const int64_t num_stages = (red_len + BK - 1) / BK;
+        if (num_stages > 0) {
+            Pipe::prologue(*this);
+            int64_t s = 0;
+            for (; s + Pipe::CYCLE <= num_stages; s += Pipe::CYCLE) full_cycle<0>(s, acc);
+            steps_from<0>(s, num_stages - s, acc);  // fewer than CYCLE steps remain
+            wait_vmcnt<0>();                         // the trailing zero-page loads
+        }
+        block_barrier();  // every wave is done reading the slabs; no load is in flight any more
     }
 };
 
-template <typename T, int KIND, int EPI>
+template <typename T, int KIND, int EPI, typename Pipe>
 __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmParams P) {
-    using K = Kernel<T, KIND, EPI>;
+    using K = Kernel<T, KIND, EPI, Pipe>;
     constexpr int PV = 8;
     constexpr int BN_OUT = K::BN_OUT;
 
@@ -262,10 +346,10 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 
     // ---- operand load plans ----
     if constexpr (KIND == XMA_GEMM_MT) {
-        setup_kstrided(k.la, k.wave, k.lane, A + m_begin * P.lda + tile_i0, P.lda, P.n - tile_i0);
-        setup_kstrided(k.lb, k.wave, k.lane, B + m_begin * P.ldb + n0, P.ldb, P.k - n0);
+        k.la.setup_kstrided(k.wave, k.lane, A + m_begin * P.lda + tile_i0, P.lda, P.n - tile_i0);
+        k.lb.setup_kstrided(k.wave, k.lane, B + m_begin * P.ldb + n0, P.ldb, P.k - n0);
     } else {
-        setup_kcontig(k.la, k.wave, k.lane, [&](int r) -> const T* {
+        k.la.setup_kcontig(k.wave, k.lane, [&](int r) -> const T* {
             const int64_t p = m_begin + r;
             if (p >= m_end) return nullptr;
             const int64_t src = P.in_index ? source_row(P, p) : p;
@@ -273,7 +357,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         });
         const T* W = B + (int64_t)expert * P.b_expert_stride;
         if constexpr (KIND == XMA_GEMM_TN) {
-            setup_kcontig(k.lb, k.wave, k.lane, [&](int r) -> const T* {
+            k.lb.setup_kcontig(k.wave, k.lane, [&](int r) -> const T* {
                 int64_t n;
                 if constexpr (EPI == XMA_EPI_SWIGLU) {
                     const int64_t half = P.n / 2;
@@ -287,9 +371,10 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                 return W + n * P.ldb;
             });
         } else {
-            setup_kstrided(k.lb, k.wave, k.lane, W + n0, P.ldb, P.n - n0);
+            k.lb.setup_kstrided(k.wave, k.lane, W + n0, P.ldb, P.n - n0);
         }
     }
+    k.init_fragments();
 
     f32x16_t acc[MI][NI];
 #pragma unroll
@@ -299,23 +384,9 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
 
-    // ---- pipelined main loop: the stage count is rounded up to a multiple of NS with all-zero stages ----
-    const int64_t num_stages = (k.red_len + BK - 1) / BK;
-    if (num_stages > 0) {
-        k.template issue<0>(0);
-        k.template issue<1>(1);
-        k.template issue<2>(2);
-        for (int64_t s = 0; s < num_stages; s += NS) {
-            k.template step<0>(s, acc);
-            k.template step<1>(s + 1, acc);
-            k.template step<2>(s + 2, acc);
-            k.template step<3>(s + 3, acc);
-        }
-        wait_vmcnt<0>();  // the trailing zero-page loads
-    }
-    block_barrier();  // every wave is done reading the stages; no load is in flight any more
+    k.run(acc);
 
-    // ---- epilogue: accumulators -> LDS (stage array mi holds the 64 tile rows {wr*128 + mi*32 + 0..31}) -> HBM ----
+    // ---- epilogue: accumulators -> LDS (slab mi holds the 64 tile rows {wr*128 + mi*32 + 0..31}) -> HBM ----
     // MFMA result element r of lane l: tile column 8*(r/4) + 4*(l/32) + r%4 (+32*ni), tile row l%32 (+32*mi).
     // A 512-byte LDS row holds 32 chunks of 8 columns; chunk c of buffer row br sits at c ^ (br & 31).
     {
@@ -334,10 +405,10 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                 }
             }
         };
-        write_rows(stage_ptr<0>(), acc[0]);
-        write_rows(stage_ptr<1>(), acc[1]);
-        write_rows(stage_ptr<2>(), acc[2]);
-        write_rows(stage_ptr<3>(), acc[3]);
+        write_rows(slab<0>(), acc[0]);
+        write_rows(slab<1>(), acc[1]);
+        write_rows(slab<2>(), acc[2]);
+        write_rows(slab<3>(), acc[3]);
     }
     __syncthreads();
 
@@ -375,7 +446,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                             Elem<T>::unpack(chunk_at(cc), u);
                             Elem<T>::unpack(chunk_at(cc + HALF_CHUNKS), g);
 #pragma unroll
-                            for (int q = 0; q < PV; ++q) o[q] = u[q] * (g[q] * sigmoid_f32(g[q]));
+                            for (int q = 0; q < PV; ++q) o[q] = u[q] * (g[q] * sigmoid_fast(g[q]));
                             *reinterpret_cast<uint4*>(C + orow * P.ldc + j) = Elem<T>::pack(o);
                         }
                     }
@@ -389,7 +460,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                         Elem<T>::unpack(chunk_at(cc), d);
 #pragma unroll
                         for (int q = 0; q < PV; ++q) {
-                            const float sg = sigmoid_f32(g[q]);
+                            const float sg = sigmoid_fast(g[q]);
                             dg[q] = d[q] * u[q] * (sg + g[q] * sg * (1.0f - sg));
                             du[q] = d[q] * g[q] * sg;
                         }
@@ -400,13 +471,13 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             }
         }
     };
-    store_rows(stage_ptr<0>(), 0);
-    store_rows(stage_ptr<1>(), 1);
-    store_rows(stage_ptr<2>(), 2);
-    store_rows(stage_ptr<3>(), 3);
+    store_rows(slab<0>(), 0);
+    store_rows(slab<1>(), 1);
+    store_rows(slab<2>(), 2);
+    store_rows(slab<3>(), 3);
 }
 
-template <typename T, int KIND, int EPI>
+template <typename T, int KIND, int EPI, typename Pipe>
 static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
     GemmParams P;
     fill_params(a, P);
@@ -430,21 +501,22 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
                            ws + 4, ws + 4 + rt, ws);
     }
     XMA_REQUIRE(grid < ((int64_t)1 << 31), "xma_grouped_gemm: %lld tiles exceed the grid limit", (long long)grid);
-    hipLaunchKernelGGL((grouped_gemm_dma_kernel<T, KIND, EPI>), dim3((unsigned)grid), dim3(THREADS), 0, stream, P);
+    hipLaunchKernelGGL((grouped_gemm_dma_kernel<T, KIND, EPI, Pipe>), dim3((unsigned)grid), dim3(THREADS), 0, stream, P);
     return check_launch("xma_grouped_gemm");
 }
 
 template <typename T>
 static int dispatch(const xma_grouped_gemm_args& a, hipStream_t stream) {
+    using Pipe = Pipe32x4;
     switch (a.kind) {
         case XMA_GEMM_TN:
-            if (a.epilogue == XMA_EPI_SWIGLU) return launch<T, XMA_GEMM_TN, XMA_EPI_SWIGLU>(a, stream);
-            return launch<T, XMA_GEMM_TN, XMA_EPI_NONE>(a, stream);
+            if (a.epilogue == XMA_EPI_SWIGLU) return launch<T, XMA_GEMM_TN, XMA_EPI_SWIGLU, Pipe>(a, stream);
+            return launch<T, XMA_GEMM_TN, XMA_EPI_NONE, Pipe>(a, stream);
         case XMA_GEMM_NN:
-            if (a.epilogue == XMA_EPI_SWIGLU_BWD) return launch<T, XMA_GEMM_NN, XMA_EPI_SWIGLU_BWD>(a, stream);
-            return launch<T, XMA_GEMM_NN, XMA_EPI_NONE>(a, stream);
+            if (a.epilogue == XMA_EPI_SWIGLU_BWD) return launch<T, XMA_GEMM_NN, XMA_EPI_SWIGLU_BWD, Pipe>(a, stream);
+            return launch<T, XMA_GEMM_NN, XMA_EPI_NONE, Pipe>(a, stream);
         default:
-            return launch<T, XMA_GEMM_MT, XMA_EPI_NONE>(a, stream);
+            return launch<T, XMA_GEMM_MT, XMA_EPI_NONE, Pipe>(a, stream);
     }
 }
 

@@ -455,6 +455,12 @@ def group_bwd_W(
         assert x_index.numel() == rows
     else:
         assert X.size(0) == rows
+    if x_index is not None and X.dtype != torch.float32 and DW.stride(1) == 1:
+        # the LDS-DMA kernel walks the routed rows with a fixed stride, so 16-bit activations are
+        # gathered once (an HBM-bound pass two orders of magnitude cheaper than the GEMM)
+        gathered = torch.empty(rows, X.size(1), dtype=X.dtype, device=X.device)
+        group(X, x_index, gathered, None, x_fan_out)
+        X, x_index, x_fan_out = gathered, None, 1
     common = dict(
         kind=nat.GEMM_MT,
         epilogue=nat.EPI_NONE,
