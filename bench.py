@@ -26,6 +26,16 @@ if ROOT not in sys.path:
 PEAK_BF16_FLOPS = 2.5e15
 PEAK_HBM_BYTES = 8.0e12
 
+# HBM-side bytes per launch of the grouped GEMM kernels at this workload, from rocprofv3 FETCH_SIZE (x 2.0) and
+# WRITE_SIZE (x 1.0), the factors a plain 1 GiB copy gives; see profiles/moe_c2_bench_rocprofv3.txt
+MEASURED_TRAFFIC_BYTES = {
+    "xma_grouped_gemm/MT": (2064572 * 2.0 + 1376256) * 1024,
+    "xma_grouped_gemm/TN+swiglu": (3725129 * 2.0 + 1376256) * 1024,
+    "xma_grouped_gemm/TN": (2055901 * 2.0 + 131072) * 1024,
+    "xma_grouped_gemm/NN+swiglu_bwd": (2300666 * 2.0 + 917504) * 1024,
+    "xma_grouped_gemm/NN": (3891177 * 2.0 + 131072) * 1024,
+}
+
 WORKLOAD = {
     "workload": "Mixtral-shaped MoE layer, forward+backward",
     "tokens": 8192,
@@ -45,6 +55,11 @@ def _parse() -> argparse.Namespace:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    ap.add_argument(
+        "--copy-probe",
+        action="store_true",
+        help="also run one plain 1 GiB device copy, the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE",
+    )
     return ap.parse_args()
 
 
@@ -119,6 +134,13 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
 
+    if args.copy_probe:
+        src = torch.empty(1 << 29, dtype=dt, device=dev).normal_()  # 1 GiB read, 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     timeline = _native.Timeline()
     _native.set_timeline(timeline)
     t0 = time.perf_counter()
@@ -142,6 +164,7 @@ def main() -> int:
             "ms_per_step": round(row["ms"] / args.steps, 4),
         }
         if row["flops"] > 0:
+            entry["flops_per_launch"] = row["flops"] / row["launches"]
             entry["tflops"] = round(row["flops"] / row["ms"] / 1e9, 2)
             entry["frac_of_bf16_peak"] = round(row["flops"] / (row["ms"] * 1e-3) / PEAK_BF16_FLOPS, 4)
         elif row["bytes"] > 0:
@@ -158,7 +181,8 @@ def main() -> int:
             "peak": PEAK_BF16_FLOPS / 1e12,
             "unit": "TFLOP/s",
             "frac": dominant["frac_of_bf16_peak"],
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(dominant["kernel"]),
+            "algorithmic_flops_per_launch": dominant["flops_per_launch"],
         }
     else:
         roofline = {
