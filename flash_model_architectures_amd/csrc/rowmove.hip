@@ -8,6 +8,17 @@ namespace xma {
 
 constexpr int kRowsPerIter = 4;
 
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+
+// Streaming accesses: each byte is touched once, so keep it from displacing reusable lines in the caches.
+__device__ __forceinline__ uint4 load_stream(const void* p) {
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void store_stream(void* p, const uint4& v) {
+    __builtin_nontemporal_store(u32x4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4_t*>(p));
+}
+
 enum RowMode { kGather = 0, kScatter = 1 };
 
 // 16-byte path: cols is a multiple of Elem<T>::kPerVec, strides keep rows 16-byte aligned.
@@ -34,7 +45,7 @@ __global__ __launch_bounds__(256) void move_rows_vec_kernel(const T* __restrict_
             uint4 v[kRowsPerIter];
 #pragma unroll
             for (int j = 0; j < kRowsPerIter; ++j)
-                v[j] = *reinterpret_cast<const uint4*>(src + srow[j] * ld_src + (int64_t)c * PV);
+                v[j] = load_stream(src + srow[j] * ld_src + (int64_t)c * PV);
 #pragma unroll
             for (int j = 0; j < kRowsPerIter; ++j) {
                 if constexpr (COEFF) {
@@ -44,7 +55,7 @@ __global__ __launch_bounds__(256) void move_rows_vec_kernel(const T* __restrict_
                     for (int q = 0; q < PV; ++q) f[q] *= scale[j];
                     v[j] = Elem<T>::pack(f);
                 }
-                if (r0 + j < rows) *reinterpret_cast<uint4*>(dst + drow[j] * ld_dst + (int64_t)c * PV) = v[j];
+                if (r0 + j < rows) store_stream(dst + drow[j] * ld_dst + (int64_t)c * PV, v[j]);
             }
         }
     }
