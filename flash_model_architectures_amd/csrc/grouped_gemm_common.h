@@ -14,6 +14,10 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // 16 bytes moved
 constexpr int kNumXcd = 8;     // accelerator complex dies, each with a private L2
 constexpr int kBandTiles = 4;  // row tiles per band of the tile walk
 
+#ifndef XMA_SPREAD
+#define XMA_SPREAD(KIND) ((KIND) == XMA_GEMM_MT)
+#endif
+
 // ---- kernel arguments -----------------------------------------------------------------------------
 struct GemmParams {
     const void* a;
@@ -75,28 +79,45 @@ static __global__ __launch_bounds__(1024) void build_row_tiles_kernel(const int3
 }
 
 
-// Work-group -> (row tile, column tile).  Work-groups are dealt round-robin to the XCDs, so the
-// block index is first renumbered to give every XCD a contiguous range of tiles; tiles are then
-// walked in bands of kBandTiles row tiles x all column tiles, row tile fastest, so that work-groups
-// running at the same time share A row panels and B column panels in their XCD's L2.
-// Returns false when this work-group has no tile.
+// Work-group -> (row tile, column tile).  Tiles are numbered in bands of kBandTiles row tiles x all column
+// tiles, row tile fastest, so that work-groups running at the same time share A row panels and B column
+// panels.  The hardware deals work-groups round-robin to the XCDs (block b runs on XCD b % 8, as that XCD's
+// b / 8-th block; checked on the device), and each XCD has a private L2, so neighbouring tiles must go to
+// the same XCD.  Two ways to deal the tiles:
+//   SPREAD = false: XCD x takes the x-th of eight equal contiguous ranges of the tile sequence (ranges may
+//     cut a band).  Balanced to one tile when every tile costs the same (row-grouped kinds).
+//   SPREAD = true: XCD x takes whole bands x, x+8, x+16, ...; spreads a run of expensive bands (the
+//     weight-gradient tiles of an overloaded expert) over all XCDs.
+// `row_tiles` is the number of row tiles actually present.  Returns false when this work-group has no tile.
+template <bool SPREAD>
 __device__ __forceinline__ bool locate_tile(int row_tiles, int col_tiles, int& row_tile, int& col_tile) {
-    const int nwg = gridDim.x;  // a multiple of kNumXcd
-    const int pid = (blockIdx.x % kNumXcd) * (nwg / kNumXcd) + blockIdx.x / kNumXcd;
-    const int band = pid / (kBandTiles * col_tiles);
+    const int xcd = blockIdx.x % kNumXcd;
+    const int local = blockIdx.x / kNumXcd;
+    const int per_band = kBandTiles * col_tiles;
+    int band, in_band;
+    if constexpr (SPREAD) {
+        band = (local / per_band) * kNumXcd + xcd;
+        in_band = local % per_band;
+    } else {
+        const int total = row_tiles * col_tiles;
+        const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
+        const int tile = xcd * per_xcd + local;
+        if (local >= per_xcd || tile >= total) return false;
+        band = tile / per_band;
+        in_band = tile - band * per_band;
+    }
     const int band_first = band * kBandTiles;
     if (band_first >= row_tiles) return false;
     const int band_rows = row_tiles - band_first < kBandTiles ? row_tiles - band_first : kBandTiles;
-    const int in_band = pid - band * (kBandTiles * col_tiles);
     row_tile = band_first + in_band % band_rows;
     col_tile = in_band / band_rows;
     return col_tile < col_tiles;
 }
 
-// number of work-groups that covers `row_tiles` x `col_tiles` under locate_tile()
+// number of work-groups that covers up to `row_tiles` x `col_tiles` under either dealing of locate_tile()
 inline int64_t grid_for_tiles(int64_t row_tiles, int64_t col_tiles) {
-    const int64_t tiles = ceil_div(row_tiles, kBandTiles) * kBandTiles * col_tiles;
-    return ceil_div(tiles, kNumXcd) * kNumXcd;
+    const int64_t bands = ceil_div(row_tiles, kBandTiles);
+    return ceil_div(bands, kNumXcd) * kNumXcd * kBandTiles * col_tiles;
 }
 
 inline int64_t max_row_tiles(int64_t rows, int E, int BM) { return rows / BM + E; }

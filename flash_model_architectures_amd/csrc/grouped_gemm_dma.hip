@@ -321,7 +321,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 
     const int row_tiles = KIND == XMA_GEMM_MT ? P.row_tiles_max * P.num_experts : P.tile_count[0];
     int row_tile, col_tile;
-    if (!locate_tile(row_tiles, P.col_tiles, row_tile, col_tile)) return;
+    if (!locate_tile<XMA_SPREAD(KIND)>(row_tiles, P.col_tiles, row_tile, col_tile)) return;
 
     const T* A = reinterpret_cast<const T*>(P.a);
     const T* B = reinterpret_cast<const T*>(P.b);
