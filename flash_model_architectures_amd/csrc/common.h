@@ -81,8 +81,11 @@ struct Elem<bf16_t> {
             out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
         }
     }
+    // two floats -> packed bf16 pair, round to nearest even: one v_cvt_pk_bf16_f32 on gfx950
     __device__ static __forceinline__ uint32_t pack2(float a, float b) {
-        return float_to_bf16_bits(a) | (float_to_bf16_bits(b) << 16);
+        typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+        typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, bf16x2_t));
     }
     __device__ static __forceinline__ uint4 pack(const float* in) {
         return make_uint4(pack2(in[0], in[1]), pack2(in[2], in[3]), pack2(in[4], in[5]), pack2(in[6], in[7]));
@@ -127,7 +130,9 @@ __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + ex
 
 // sigmoid from the hardware exp2 and reciprocal (a few ulp in fp32): for results that are rounded to a
 // 16-bit type anyway
-__device__ __forceinline__ float sigmoid_fast(float x) { return __frcp_rn(1.0f + __expf(-x)); }
+__device__ __forceinline__ float sigmoid_fast(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+}
 
 // ---- wave64 primitives ------------------------------------------------------------------------
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (kWaveSize - 1)); }

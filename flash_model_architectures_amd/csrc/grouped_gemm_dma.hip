@@ -4,12 +4,17 @@
 // reduction index is strided in HBM are fetched in their HBM layout and transposed by the LDS read
 // itself (ds_read_b64_tr_b16).
 //
-// Tile 256 x 256 per work-group, 8 waves as 2 x 4, each wave 128 x 64 (4 x 2 MFMA 32x32x16 tiles).
+// Tile 256 x 256 per work-group, 4 waves as 2 x 2, one wave per SIMD with the whole 512-register budget:
+// each wave owns 128 x 128 (4 x 4 MFMA 32x32x16 tiles, 256 accumulator registers).  A wave that is alone
+// on its SIMD has nobody to hide its stalls, so the main loop is software-pipelined by hand: the fragments
+// of reduction block k+1 are read from LDS while block k is multiplied, DMA loads are dealt out a few per
+// block, and the instruction scheduler is told how to interleave the three streams.
 //
-// LDS is a pool of four 32 KiB slabs; the pipeline policy Pipe32x4 keeps four stages of 32 reduction
-// elements in them, one slab each (A tile | B tile), with three stages of loads in flight.  (A variant
-// with 64-deep blocks rotating through five slabs, so that every DMA instruction asks for whole 128-byte
-// lines, measured the same or slower on the layer's shapes and was dropped.)
+// What bounds the loop (measured): a compute unit pulls a 256 x 256 tile's operands from L2 at
+// 128 FLOP per byte, and the L2 delivers whole 128-byte lines about 1.5 x faster than half lines.  So
+// K-contiguous operands are staged 64 reduction elements at a time (128-byte rows); see Ring64x5.
+//
+// LDS is a pool of five 32 KiB slabs (all 160 KiB of the compute unit).
 // Tile layouts inside a slab:
 //   K-contiguous operand (A in TN/NN, W in TN): [256 tile rows][BK k]; the 16-byte chunks of a row are
 //     XOR-swizzled by the row number so that the 16 rows a quarter-wave reads in one ds_read_b128 cover all
@@ -20,13 +25,25 @@
 // A DMA load writes lane l's 16 bytes at (wave-uniform LDS base) + 16*l, so the swizzles are applied
 // by choosing which HBM chunk each lane fetches.  Masked rows / reduction tails are fetched from a
 // 16-byte page of zeros, which keeps every lane active and the outstanding-load count uniform.
+#include <type_traits>
+
 #include "grouped_gemm_common.h"
+
+#ifndef XMA_PIPE_TN
+#define XMA_PIPE_TN Ring64x5
+#endif
+#ifndef XMA_PIPE_NN
+#define XMA_PIPE_NN Ring64x5
+#endif
+#ifndef XMA_PIPE_MT
+#define XMA_PIPE_MT Ring32x5
+#endif
 
 namespace xma {
 namespace dma {
 
-constexpr int BM = 256, BN = 256, THREADS = 512;
-constexpr int WAVES_N = 4, WM = 128, WN = 64, MI = WM / 32, NI = WN / 32;
+constexpr int BM = 256, BN = 256, THREADS = 256, NUM_WAVES = THREADS / 64;
+constexpr int WAVES_N = 2, WM = 128, WN = 128, MI = WM / 32, NI = WN / 32;
 constexpr int SLAB_BYTES = 32768;
 static_assert(BM == BN, "both operands use the same tile height");
 
@@ -34,16 +51,18 @@ __shared__ __attribute__((aligned(1024))) char slab0[SLAB_BYTES];
 __shared__ __attribute__((aligned(1024))) char slab1[SLAB_BYTES];
 __shared__ __attribute__((aligned(1024))) char slab2[SLAB_BYTES];
 __shared__ __attribute__((aligned(1024))) char slab3[SLAB_BYTES];
+__shared__ __attribute__((aligned(1024))) char slab4[SLAB_BYTES];
 
 // The slabs are distinct arrays on purpose: the compiler can then prove that a fragment read of
 // one slab does not alias the DMA writes still in flight to the others, and does not drain them.
 template <int I>
 __device__ __forceinline__ char* slab() {
-    static_assert(I >= 0 && I < 4, "slab index");
+    static_assert(I >= 0 && I < 5, "slab index");
     if constexpr (I == 0) return slab0;
     if constexpr (I == 1) return slab1;
     if constexpr (I == 2) return slab2;
-    return slab3;
+    if constexpr (I == 3) return slab3;
+    return slab4;
 }
 
 __device__ __attribute__((aligned(16))) uint32_t g_zero_page[4];  // zero-initialised
@@ -61,6 +80,15 @@ __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N < 64, "vmcnt range");
     compiler_fence();
     __builtin_amdgcn_s_waitcnt((N & 0xF) | (7 << 4) | (0xF << 8) | ((N >> 4) << 14));
+    compiler_fence();
+}
+
+// s_waitcnt on the vector-memory counter and for every LDS read of this wave (lgkmcnt = 0)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_and_lds() {
+    static_assert(N >= 0 && N < 64, "vmcnt range");
+    compiler_fence();
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
     compiler_fence();
 }
 
@@ -85,7 +113,7 @@ struct Geometry {
     static constexpr int CPR = BK / 8;            // 16-byte chunks per K-contiguous row
     static constexpr int ROW_BYTES = BK * 2;
     static constexpr int ROWS_PER_LOAD = 64 / CPR;  // tile rows one DMA instruction covers
-    static constexpr int LOADS = BK / 16;         // DMA instructions per wave, operand and stage
+    static constexpr int LOADS = BK / 2 / NUM_WAVES;  // DMA instructions per wave, operand and stage
     static constexpr int TILE_BYTES = BM * BK * 2;
     static_assert(BK == 32 || BK == 64, "stage depth");
 
@@ -123,82 +151,156 @@ __device__ __forceinline__ u32x4_t read_fragment(const char* slab_base, int offs
 }
 
 // ---- per-thread DMA plan of one operand ---------------------------------------------------------------
-template <typename T, int BK>
+// DMA instruction i of wave w fills the 1 KiB block (i * NUM_WAVES + w) of the operand's LDS tile:
+//   K-contiguous tile: tile rows [R * (i * NUM_WAVES + w), +R), R = ROWS_PER_LOAD; lane l -> row + l / CPR,
+//     physical chunk l % CPR (the logical chunk it fetches is the XOR-swizzled one, and because R * NUM_WAVES
+//     is a multiple of the swizzle period it is the same for every i);
+//   K-strided tile: k rows {2 * (i * NUM_WAVES + w), +1}; lane l -> k row + l / 32, physical chunk l % 32.
+// Three address plans:
+//   ROWS     one pointer per instruction (rows that are gathered through an index table or end anywhere),
+//   UNIFORM  K-contiguous rows at a constant stride, with one extra jump in the middle of the tile
+//            (the up|gate halves of a fused SwiGLU weight tile): one pointer, the rest is scalar arithmetic,
+//   STRIDED  K-strided tile: one pointer, constant stride between instructions.
+enum LoadPlan { PLAN_ROWS, PLAN_UNIFORM, PLAN_STRIDED };
+
+template <typename T, int BK, LoadPlan PLAN>
 struct OperandLoads {
-    static constexpr int LOADS = Geometry<BK>::LOADS;
-    const T* ptr[LOADS];  // HBM address of this lane's chunk in stage 0 (or the zero page)
-    int64_t step;         // elements to advance per stage
-    int32_t red[LOADS];   // reduction index covered by the lane in stage 0 (chunk start or k row)
-    bool valid[LOADS];    // false: always the zero page (row / column outside the operand)
-    int lds_off[LOADS];   // byte offset of the wave's 1 KiB destination inside the operand's LDS tile
+    using G = Geometry<BK>;
+    static constexpr int LOADS = G::LOADS;
+    static constexpr int RED_STRIDE = PLAN == PLAN_STRIDED ? 2 * NUM_WAVES : 0;  // reduction rows between i and i+1
+    const T* ptr[PLAN == PLAN_ROWS ? LOADS : 1];  // HBM address of this lane's chunk in stage 0
+    bool valid[PLAN == PLAN_STRIDED ? 1 : LOADS];  // false: always the zero page (row / column outside the operand)
+    int64_t load_stride, mid_jump;  // UNIFORM / STRIDED: elements from instruction i to i+1; UNIFORM: extra at LOADS/2
+    int64_t step;                   // elements to advance per stage
+    int32_t red0;                   // reduction index covered by the lane in stage 0, instruction 0
+    int wave_lds;                   // byte offset of the wave's first 1 KiB block inside the operand's LDS tile
 
-    // K-contiguous layout: DMA instruction i of wave w fills tile rows [R*(8i + w), +R), R = ROWS_PER_LOAD:
-    // lane l -> row + l/CPR, physical chunk l%CPR.  row_fn(tile row) returns the HBM row base or nullptr.
+    __device__ static __forceinline__ const T* zero_page() { return reinterpret_cast<const T*>(g_zero_page); }
+
+    // ROWS: row_fn(tile row) returns the HBM row base or nullptr.
     template <typename RowFn>
-    __device__ __forceinline__ void setup_kcontig(int wave, int lane, RowFn row_fn) {
-        using G = Geometry<BK>;
+    __device__ __forceinline__ void setup_rows(int wave, int lane, RowFn row_fn) {
+        static_assert(PLAN == PLAN_ROWS, "plan");
+        const int chunk = (lane % G::CPR) ^ G::swizzle(wave * G::ROWS_PER_LOAD + lane / G::CPR);
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
-            const int row0 = (i * 8 + wave) * G::ROWS_PER_LOAD;
-            const int row = row0 + lane / G::CPR;
-            const int chunk = (lane % G::CPR) ^ G::swizzle(row);  // logical chunk stored at physical position
-            const T* base = row_fn(row);
+            const T* base = row_fn((i * NUM_WAVES + wave) * G::ROWS_PER_LOAD + lane / G::CPR);
             valid[i] = base != nullptr;
-            ptr[i] = valid[i] ? base + chunk * 8 : reinterpret_cast<const T*>(g_zero_page);
-            red[i] = chunk * 8;
-            lds_off[i] = row0 * G::ROW_BYTES;
+            ptr[i] = valid[i] ? base + chunk * 8 : zero_page();
         }
+        red0 = chunk * 8;
         step = BK;
+        wave_lds = wave * 1024;
     }
 
-    // K-strided layout: DMA instruction i of wave w fills k rows {2*(8i + w), +1}: lane l -> k row + l/32,
-    // physical chunk l%32.  `base` points at (reduction row 0, first tile column); `cols_left` = number of
-    // valid columns from there; ld = row stride.
-    __device__ __forceinline__ void setup_kstrided(int wave, int lane, const T* base, int64_t ld, int64_t cols_left) {
+    // UNIFORM: tile row r lives at base + r * ld (+ jump for r >= 128); rows_fn(tile row) says whether it exists.
+    template <typename ValidFn>
+    __device__ __forceinline__ void setup_uniform(int wave, int lane, const T* base, int64_t ld, int64_t jump,
+                                                  ValidFn valid_fn) {
+        static_assert(PLAN == PLAN_UNIFORM, "plan");
+        const int row = wave * G::ROWS_PER_LOAD + lane / G::CPR;
+        const int chunk = (lane % G::CPR) ^ G::swizzle(row);
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int krow0 = (i * 8 + wave) * 2;
-            const int krow = krow0 + (lane >> 5);
-            const int chunk = (lane & 31) ^ ((krow & 3) << 2);
-            valid[i] = chunk * 8 < cols_left;
-            ptr[i] = valid[i] ? base + (int64_t)krow * ld + chunk * 8 : reinterpret_cast<const T*>(g_zero_page);
-            red[i] = krow;
-            lds_off[i] = krow0 * (BN * 2);
-        }
+        for (int i = 0; i < LOADS; ++i) valid[i] = valid_fn(i * NUM_WAVES * G::ROWS_PER_LOAD + row);
+        ptr[0] = base + row * ld + chunk * 8;
+        load_stride = NUM_WAVES * G::ROWS_PER_LOAD * ld;
+        mid_jump = jump;
+        red0 = chunk * 8;
+        step = BK;
+        wave_lds = wave * 1024;
+    }
+
+    // STRIDED: `base` points at (reduction row 0, first tile column); `cols_left` = number of valid columns
+    // from there; ld = row stride.
+    __device__ __forceinline__ void setup_strided(int wave, int lane, const T* base, int64_t ld, int64_t cols_left) {
+        static_assert(PLAN == PLAN_STRIDED, "plan");
+        const int krow = wave * 2 + (lane >> 5);
+        const int chunk = (lane & 31) ^ ((krow & 3) << 2);  // 2 * NUM_WAVES is a multiple of 4: same for every i
+        valid[0] = chunk * 8 < cols_left;
+        ptr[0] = valid[0] ? base + (int64_t)krow * ld + chunk * 8 : zero_page();
+        load_stride = 2 * NUM_WAVES * ld;
+        mid_jump = 0;
+        red0 = krow;
         step = (int64_t)BK * ld;
+        wave_lds = wave * 1024;
     }
 
-    // Issue this wave's loads for the stage `stage` into the tile at slab_base + tile_off.
+    // Issue this wave's loads I0 <= i < I1 of the stage `stage` into the tile at slab_base + tile_off.
+    template <int I0, int I1>
     __device__ __forceinline__ void issue(char* slab_base, int tile_off, int64_t stage, int64_t red_len) const {
+        const int64_t red_left = red_len - stage * BK;  // wave-uniform
+        const int64_t stage_off = stage * step;
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const bool ok = valid[i] && (stage * BK + red[i] < red_len);
-            const T* src = ok ? ptr[i] + stage * step : reinterpret_cast<const T*>(g_zero_page);
-            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(src),
-                                             XMA_LDS(slab_base + (tile_off + lds_off[i])), 16, 0, 0);
+        for (int i = I0; i < I1; ++i) {
+            const bool ok = valid[PLAN == PLAN_STRIDED ? 0 : i] && (red0 + i * RED_STRIDE < red_left);
+            const T* p;
+            if constexpr (PLAN == PLAN_ROWS) p = ptr[i] + stage_off;
+            else p = ptr[0] + (stage_off + i * load_stride + (i >= LOADS / 2 ? mid_jump : 0));
+            // computed for every lane and then selected: a branch around the load would make the number of
+            // loads in flight differ between waves
+            asm("" : "+v"(p));
+            p = ok ? p : zero_page();
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(p),
+                                             XMA_LDS(slab_base + (tile_off + i * NUM_WAVES * 1024 + wave_lds)), 16, 0, 0);
         }
     }
 };
 
 // ---- pipeline policies --------------------------------------------------------------------------------------
-// A policy names, for every position P of its unrolled cycle, the slab and offset of the A and B tiles
-// that step P multiplies, what the step loads, and how many younger DMA instructions may stay in flight
-// when the step starts.
-struct Pipe32x4 {
-    static constexpr int BK = 32, CYCLE = 4;
-    static constexpr int WAIT = 2 * 2 * Geometry<BK>::LOADS;  // two younger stages, two operands each
+// A policy says where the tiles of stage j live, which loads the step at cycle position P issues in
+// each of its phases (one phase = 16 reduction elements), and how many loads may still be in flight when
+// the step reaches its barrier.  Loads are spread evenly over the phases: the texture path of a compute
+// unit takes about sixteen cycles per DMA instruction and a wave that issues into a full queue stalls,
+// matrix instructions included.
+//
+// Ring32x5: stage j of 32 reduction elements lives in slab j % 5 (A tile | B tile).  At a step's barrier
+// the next stage has landed and three more are in flight; the step's own slab then takes stage s+5:
+// its A tile during the rest of this step, its B tile during the first phase of the next step.
+struct Ring32x5 {
+    static constexpr int BK = 32, CYCLE = 5, KK = 2;
+    static constexpr int L = Geometry<BK>::LOADS;
+    static constexpr int PHASE_LOADS = L;
+    static constexpr int WAIT = 6 * L;           // loads that may stay in flight at a step's barrier
+    static constexpr int PROLOGUE_WAIT = 7 * L;  // ... and when the first stage is needed
     template <int P> struct At {
         static constexpr int A_SLAB = P, A_OFF = 0, B_SLAB = P, B_OFF = Geometry<BK>::TILE_BYTES;
     };
     template <typename K> __device__ static __forceinline__ void prologue(K& k) {
-        k.template issue_a<0>(0); k.template issue_b<0>(0);
-        k.template issue_a<1>(1); k.template issue_b<1>(1);
-        k.template issue_a<2>(2); k.template issue_b<2>(2);
+        k.template issue_a<0, 0, L>(0); k.template issue_b<0, 0, L>(0);
+        k.template issue_a<1, 0, L>(1); k.template issue_b<1, 0, L>(1);
+        k.template issue_a<2, 0, L>(2); k.template issue_b<2, 0, L>(2);
+        k.template issue_a<3, 0, L>(3); k.template issue_b<3, 0, L>(3);
+        k.template issue_a<4, 0, L>(4);
     }
-    // step s refills the slab that step s-1 released with stage s+3
-    template <int P, typename K> __device__ static __forceinline__ void refill(K& k, int64_t s) {
-        k.template issue_a<(P + 3) % CYCLE>(s + 3);
-        k.template issue_b<(P + 3) % CYCLE>(s + 3);
+    template <int P, int PH, typename K> __device__ static __forceinline__ void issue_phase(K& k, int64_t s) {
+        if constexpr (PH == 0) k.template issue_b<(P + 4) % CYCLE, 0, L>(s + 4);
+        else k.template issue_a<P, 0, L>(s + 5);
+    }
+};
+
+// Ring64x5: stage j of 64 reduction elements keeps its A tile in slab (2j) % 5 and its B tile in slab
+// (2j + 1) % 5, so every DMA instruction of a K-contiguous operand asks for whole 128-byte lines.  At a
+// step's barrier the next stage has landed and the A tile of the one after is in flight.  The step's own
+// slabs then take the B tile of stage s+2 (half after the barrier, half in the next step's first phase)
+// and the A tile of stage s+3 (second and third phase of the next step).
+struct Ring64x5 {
+    static constexpr int BK = 64, CYCLE = 5, KK = 4;
+    static constexpr int L = Geometry<BK>::LOADS, H = L / 2;
+    static constexpr int PHASE_LOADS = H;
+    static constexpr int WAIT = L;
+    static constexpr int PROLOGUE_WAIT = L + H;
+    template <int P> struct At {
+        static constexpr int A_SLAB = (2 * P) % 5, A_OFF = 0, B_SLAB = (2 * P + 1) % 5, B_OFF = 0;
+    };
+    template <typename K> __device__ static __forceinline__ void prologue(K& k) {
+        k.template issue_a<0, 0, L>(0); k.template issue_b<0, 0, L>(0);
+        k.template issue_a<1, 0, L>(1); k.template issue_b<1, 0, H>(1);
+    }
+    template <int P, int PH, typename K> __device__ static __forceinline__ void issue_phase(K& k, int64_t s) {
+        if constexpr (PH == 0) k.template issue_b<(P + 1) % CYCLE, H, L>(s + 1);
+        else if constexpr (PH == 1) k.template issue_a<(P + 2) % CYCLE, 0, H>(s + 2);
+        else if constexpr (PH == 2) k.template issue_a<(P + 2) % CYCLE, H, L>(s + 2);
+        else k.template issue_b<(P + 2) % CYCLE, 0, H>(s + 2);
     }
 };
 
@@ -210,16 +312,18 @@ struct Kernel {
     static constexpr bool B_STRIDED = KIND != XMA_GEMM_TN;
     static constexpr int BN_OUT = EPI == XMA_EPI_SWIGLU ? BN / 2 : BN;
 
-    OperandLoads<T, BK> la, lb;
+    OperandLoads<T, BK, A_STRIDED ? PLAN_STRIDED : PLAN_ROWS> la;
+    OperandLoads<T, BK, B_STRIDED ? PLAN_STRIDED : PLAN_UNIFORM> lb;
     int64_t red_len;
     int wave, lane;
     int a_off[4], b_off[4];  // variable parts of the fragment offsets (see fragment_offsets)
+    u32x4_t fa[2][MI], fb[2][NI];  // fragments: the block being multiplied and the one being read
 
-    template <int P> __device__ __forceinline__ void issue_a(int64_t stage) {
-        la.issue(slab<Pipe::template At<P>::A_SLAB>(), Pipe::template At<P>::A_OFF, stage, red_len);
+    template <int P, int I0, int I1> __device__ __forceinline__ void issue_a(int64_t stage) {
+        la.template issue<I0, I1>(slab<Pipe::template At<P>::A_SLAB>(), Pipe::template At<P>::A_OFF, stage, red_len);
     }
-    template <int P> __device__ __forceinline__ void issue_b(int64_t stage) {
-        lb.issue(slab<Pipe::template At<P>::B_SLAB>(), Pipe::template At<P>::B_OFF, stage, red_len);
+    template <int P, int I0, int I1> __device__ __forceinline__ void issue_b(int64_t stage) {
+        lb.template issue<I0, I1>(slab<Pipe::template At<P>::B_SLAB>(), Pipe::template At<P>::B_OFF, stage, red_len);
     }
 
     // Byte offsets of this lane's fragments inside an operand tile.  Only the part that is not a
@@ -244,38 +348,77 @@ struct Kernel {
         fragment_offsets<B_STRIDED, NI>((wave % WAVES_N) * WN, b_off);
     }
 
+    // Fragments of reduction block kk of the stage held at cycle position P.
     template <int P>
-    __device__ __forceinline__ void compute(f32x16_t (&acc)[MI][NI]) {
+    __device__ __forceinline__ void read_fragments(int kk, u32x4_t (&af)[MI], u32x4_t (&bf)[NI]) const {
         using At = typename Pipe::template At<P>;
         const char* ta = slab<At::A_SLAB>();
         const char* tb = slab<At::B_SLAB>();
 #pragma unroll
-        for (int kk = 0; kk < BK / 16; ++kk) {
-            u32x4_t af[MI], bf[NI];
+        for (int mi = 0; mi < MI; ++mi)
+            af[mi] = read_fragment<A_STRIDED>(ta, At::A_OFF + fragment_offset<A_STRIDED>(a_off, mi, kk));
 #pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-                af[mi] = read_fragment<A_STRIDED>(ta, At::A_OFF + fragment_offset<A_STRIDED>(a_off, mi, kk));
+        for (int ni = 0; ni < NI; ++ni)
+            bf[ni] = read_fragment<B_STRIDED>(tb, At::B_OFF + fragment_offset<B_STRIDED>(b_off, ni, kk));
+    }
+
+    __device__ __forceinline__ void multiply(const u32x4_t (&af)[MI], const u32x4_t (&bf)[NI], f32x16_t (&acc)[MI][NI]) {
 #pragma unroll
-            for (int ni = 0; ni < NI; ++ni)
-                bf[ni] = read_fragment<B_STRIDED>(tb, At::B_OFF + fragment_offset<B_STRIDED>(b_off, ni, kk));
+        for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-                for (int ni = 0; ni < NI; ++ni) Mma<T>::run(bf[ni], af[mi], acc[mi][ni]);
+            for (int ni = 0; ni < NI; ++ni) Mma<T>::run(bf[ni], af[mi], acc[mi][ni]);
+    }
+
+    // Asks the instruction scheduler to spread the LDS reads (and, with DMA, the loads) of one phase evenly
+    // between its MI*NI matrix instructions, so that a wave that is alone on its SIMD keeps the matrix
+    // pipe busy while its next fragments arrive.
+    template <int I = 0>
+    __device__ static __forceinline__ void interleave_phase() {
+        constexpr int MFMAS = MI * NI;
+        constexpr int READS = (A_STRIDED ? 2 : 1) * MI + (B_STRIDED ? 2 : 1) * NI;
+        constexpr int LOADS = Pipe::PHASE_LOADS;
+        constexpr int SLOTS = 8, READ_SLOTS = 6;  // the last slots of a phase issue no LDS read
+        static_assert(MFMAS % SLOTS == 0, "slots");
+        if constexpr (I < SLOTS) {
+            constexpr int R0 = I < READ_SLOTS ? (READS * I) / READ_SLOTS : READS;
+            constexpr int R1 = I + 1 < READ_SLOTS ? (READS * (I + 1)) / READ_SLOTS : READS;
+            __builtin_amdgcn_sched_group_barrier(0x008, MFMAS / SLOTS, 0);
+            if constexpr (R1 > R0) __builtin_amdgcn_sched_group_barrier(0x100, R1 - R0, 0);
+            constexpr int G = (LOADS * (I + 1)) / SLOTS - (LOADS * I) / SLOTS;
+            if constexpr (G > 0) __builtin_amdgcn_sched_group_barrier(0x020, G, 0);
+            interleave_phase<I + 1>();
         }
     }
 
-    // One pipeline step at cycle position P on stage s: wait until only the younger loads named by the
-    // policy are in flight, meet the other waves (stage s has landed for everybody and the slabs of stage
-    // s-1 are no longer read), refill the released slabs, multiply.  A step is branch-free: stages past the
-    // end of the reduction fetch the zero page, which keeps the count of loads in flight the same at every
-    // step and lets the compiler see that the loop needs no other wait on vector memory.
+    // One pipeline step at cycle position P on stage s.  On entry the fragments of the stage's first
+    // reduction block are in registers.  Every phase multiplies one block while the next block's fragments
+    // are read and a share of the loads is issued.  Before the last phase the step waits until its own LDS
+    // reads are done and the loads of stage s+1 have landed, and meets the other waves: stage s+1 is then
+    // complete for everybody and nobody reads stage s any more, so its slabs can be refilled while the last
+    // block is multiplied from registers and the first fragments of stage s+1 are read.  A step is
+    // branch-free: stages past the end of the reduction fetch the zero page, which keeps the count of loads
+    // in flight the same at every step and lets the compiler see that the loop needs no other wait on
+    // vector memory.
+    template <int P, int PH>
+    __device__ __forceinline__ void phases_before_barrier(int64_t s, f32x16_t (&acc)[MI][NI]) {
+        if constexpr (PH + 1 < Pipe::KK) {
+            Pipe::template issue_phase<P, PH>(*this, s);
+            read_fragments<P>(PH + 1, fa[(PH + 1) & 1], fb[(PH + 1) & 1]);
+            multiply(fa[PH & 1], fb[PH & 1], acc);
+            interleave_phase();
+            phases_before_barrier<P, PH + 1>(s, acc);
+        }
+    }
     template <int P>
     __device__ __forceinline__ void step(int64_t s, f32x16_t (&acc)[MI][NI]) {
-        wait_vmcnt<Pipe::WAIT>();
+        constexpr int KK = Pipe::KK;
+        phases_before_barrier<P, 0>(s, acc);
+        wait_vmcnt_and_lds<Pipe::WAIT>();
         block_barrier();
-        Pipe::template refill<P>(*this, s);
-        compute<P>(acc);
+        Pipe::template issue_phase<P, KK - 1>(*this, s);
+        read_fragments<(P + 1) % Pipe::CYCLE>(0, fa[KK & 1], fb[KK & 1]);
+        multiply(fa[(KK - 1) & 1], fb[(KK - 1) & 1], acc);
+        interleave_phase();
     }
 
     template <int P>
@@ -299,6 +442,9 @@ struct Kernel {
         const int64_t num_stages = (red_len + BK - 1) / BK;
         if (num_stages > 0) {
             Pipe::prologue(*this);
+            wait_vmcnt<Pipe::PROLOGUE_WAIT>();
+            block_barrier();
+            read_fragments<0>(0, fa[0], fb[0]);
             int64_t s = 0;
             for (; s + Pipe::CYCLE <= num_stages; s += Pipe::CYCLE) full_cycle<0>(s, acc);
             steps_from<0>(s, num_stages - s, acc);  // fewer than CYCLE steps remain
@@ -346,10 +492,10 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 
     // ---- operand load plans ----
     if constexpr (KIND == XMA_GEMM_MT) {
-        k.la.setup_kstrided(k.wave, k.lane, A + m_begin * P.lda + tile_i0, P.lda, P.n - tile_i0);
-        k.lb.setup_kstrided(k.wave, k.lane, B + m_begin * P.ldb + n0, P.ldb, P.k - n0);
+        k.la.setup_strided(k.wave, k.lane, A + m_begin * P.lda + tile_i0, P.lda, P.n - tile_i0);
+        k.lb.setup_strided(k.wave, k.lane, B + m_begin * P.ldb + n0, P.ldb, P.k - n0);
     } else {
-        k.la.setup_kcontig(k.wave, k.lane, [&](int r) -> const T* {
+        k.la.setup_rows(k.wave, k.lane, [&](int r) -> const T* {
             const int64_t p = m_begin + r;
             if (p >= m_end) return nullptr;
             const int64_t src = P.in_index ? source_row(P, p) : p;
@@ -357,21 +503,16 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         });
         const T* W = B + (int64_t)expert * P.b_expert_stride;
         if constexpr (KIND == XMA_GEMM_TN) {
-            k.lb.setup_kcontig(k.wave, k.lane, [&](int r) -> const T* {
-                int64_t n;
-                if constexpr (EPI == XMA_EPI_SWIGLU) {
-                    const int64_t half = P.n / 2;
-                    const int64_t j = n0 + (r % BN_OUT);
-                    if (j >= half) return nullptr;
-                    n = r < BN_OUT ? j : half + j;
-                } else {
-                    n = n0 + r;
-                    if (n >= P.n) return nullptr;
-                }
-                return W + n * P.ldb;
-            });
+            if constexpr (EPI == XMA_EPI_SWIGLU) {
+                // tile rows 0..127: weight rows n0 + r (up half); rows 128..255: P.n / 2 + n0 + r - 128 (gate half)
+                const int64_t half = P.n / 2;
+                k.lb.setup_uniform(k.wave, k.lane, W + n0 * P.ldb, P.ldb, (half - BN_OUT) * P.ldb,
+                                   [&](int r) { return n0 + (r % BN_OUT) < half; });
+            } else {
+                k.lb.setup_uniform(k.wave, k.lane, W + n0 * P.ldb, P.ldb, 0, [&](int r) { return n0 + r < P.n; });
+            }
         } else {
-            k.lb.setup_kstrided(k.wave, k.lane, W + n0, P.ldb, P.n - n0);
+            k.lb.setup_strided(k.wave, k.lane, W + n0, P.ldb, P.n - n0);
         }
     }
     k.init_fragments();
@@ -387,6 +528,54 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     k.run(acc);
 
     // ---- epilogue: accumulators -> LDS (slab mi holds the 64 tile rows {wr*128 + mi*32 + 0..31}) -> HBM ----
+    // Store phase: each thread owns one 16-byte chunk column (cc) and, per slab, the IT buffer rows
+    // tid / 32 + 8 * it.  What the rows need from HBM (scatter indices, the saved pre-activation of the
+    // SwiGLU backward) is requested in batches before it is used: the indices of all four slabs before the
+    // accumulators are packed, a slab's pre-activations before its first row is processed.
+    T* C = reinterpret_cast<T*>(P.c);
+    constexpr int C_CHUNKS = BN / PV;             // 32
+    constexpr int ROW_STEP = THREADS / C_CHUNKS;  // 8
+    constexpr int IT = 64 / ROW_STEP;             // 8
+    const int cc = tid % C_CHUNKS;
+    auto buffer_row = [&](int it) { return tid / C_CHUNKS + it * ROW_STEP; };
+    auto tile_row = [&](int mi, int br) { return (br >> 5) * 128 + mi * 32 + (br & 31); };
+
+    int32_t orow[MI][IT];  // output row of each owned row, -1: past the end of the expert's rows
+    if constexpr (KIND != XMA_GEMM_MT) {
+        // branch-free: rows past the end read the index of the expert's last row and are then marked
+        const int64_t last = m_end - 1;
+        auto fill = [&](auto index_of) {
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                for (int it = 0; it < IT; ++it) {
+                    const int64_t p = m_begin + tile_row(mi, buffer_row(it));
+                    const int32_t v = index_of(p < m_end ? p : last);
+                    orow[mi][it] = p < m_end ? v : -1;
+                }
+        };
+        if (P.out_index == nullptr) fill([&](int64_t p) { return (int32_t)p; });
+        else if (P.idx_is_i64) fill([&](int64_t p) { return (int32_t)reinterpret_cast<const int64_t*>(P.out_index)[p]; });
+        else fill([&](int64_t p) { return reinterpret_cast<const int32_t*>(P.out_index)[p]; });
+    }
+
+    // SwiGLU backward: the saved pre-activation chunks (up, gate) of the rows of slab mi, double-buffered so
+    // that slab mi+1 is on its way from HBM while slab mi is processed
+    constexpr bool SWBWD = EPI == XMA_EPI_SWIGLU_BWD;
+    u32x4_t hu[SWBWD ? 2 : 1][IT], hg[SWBWD ? 2 : 1][IT];
+    auto load_saved = [&](int mi, u32x4_t (&up)[IT], u32x4_t (&gate)[IT], const int32_t (&out_row)[IT]) {
+        // branch-free: rows / columns outside the tile's part of the operand re-read a valid chunk
+        const int64_t n = n0 + cc * PV < P.n ? n0 + cc * PV : 0;
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const int64_t p = m_begin + tile_row(mi, buffer_row(it));
+            const T* h = reinterpret_cast<const T*>(P.aux) + (out_row[it] >= 0 ? p : m_end - 1) * P.ld_aux;
+            up[it] = *reinterpret_cast<const u32x4_t*>(h + n);
+            gate[it] = *reinterpret_cast<const u32x4_t*>(h + P.n + n);
+        }
+    };
+    if constexpr (SWBWD) load_saved(0, hu[0], hg[0], orow[0]);
+
     // MFMA result element r of lane l: tile column 8*(r/4) + 4*(l/32) + r%4 (+32*ni), tile row l%32 (+32*mi).
     // A 512-byte LDS row holds 32 chunks of 8 columns; chunk c of buffer row br sits at c ^ (br & 31).
     {
@@ -412,69 +601,82 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     }
     __syncthreads();
 
-    T* C = reinterpret_cast<T*>(P.c);
-    constexpr int C_CHUNKS = BN / PV;  // 32
-    const int cc = tid % C_CHUNKS;
-    auto store_rows = [&](const char* buf, int mi) {
-#pragma unroll 1
-        for (int br = tid / C_CHUNKS; br < 64; br += THREADS / C_CHUNKS) {
-            const int r = (br >> 5) * 128 + mi * 32 + (br & 31);
-            const char* src = buf + br * (BN * 2);
-            auto chunk_at = [&](int c) { return *reinterpret_cast<const uint4*>(src + ((c ^ (br & 31)) << 4)); };
-            if constexpr (KIND == XMA_GEMM_MT) {
-                const int64_t i = tile_i0 + r, j = n0 + cc * PV;
-                if (i < P.n && j < P.k)
-                    *reinterpret_cast<uint4*>(C + (int64_t)expert * P.c_expert_stride + i * P.ldc + j) = chunk_at(cc);
-            } else {
-                const int64_t p = m_begin + r;
-                if (p >= m_end) continue;
-                const int64_t orow = P.out_index ? load_index(P.out_index, P.idx_is_i64, p) : p;
-                if constexpr (EPI == XMA_EPI_NONE) {
-                    const int64_t n = n0 + cc * PV;
-                    if (n < P.n) *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = chunk_at(cc);
-                } else if constexpr (EPI == XMA_EPI_SWIGLU) {
-                    constexpr int HALF_CHUNKS = C_CHUNKS / 2;
-                    const int64_t half_n = P.n / 2;
-                    const int64_t j = n0 + (cc % HALF_CHUNKS) * PV;
-                    if (j < half_n) {
-                        if (P.aux) {
-                            T* h = reinterpret_cast<T*>(P.aux) + p * P.ld_aux;
-                            *reinterpret_cast<uint4*>(h + (cc < HALF_CHUNKS ? j : half_n + j)) = chunk_at(cc);
-                        }
-                        if (cc < HALF_CHUNKS) {
-                            float u[PV], g[PV], o[PV];
-                            Elem<T>::unpack(chunk_at(cc), u);
-                            Elem<T>::unpack(chunk_at(cc + HALF_CHUNKS), g);
+    auto store_rows = [&](const char* buf, auto mi_tag, const int32_t (&out_row)[IT]) {
+        constexpr int mi = decltype(mi_tag)::value;
+        auto chunk_at = [&](int br, int c) {
+            return *reinterpret_cast<const u32x4_t*>(buf + br * (BN * 2) + ((c ^ (br & 31)) << 4));
+        };
+        auto to_uint4 = [](const u32x4_t& v) { return make_uint4(v[0], v[1], v[2], v[3]); };
+        if constexpr (KIND == XMA_GEMM_MT) {
+            const int64_t j = n0 + cc * PV;
+            T* out = C + (int64_t)expert * P.c_expert_stride + j;
 #pragma unroll
-                            for (int q = 0; q < PV; ++q) o[q] = u[q] * (g[q] * sigmoid_fast(g[q]));
-                            *reinterpret_cast<uint4*>(C + orow * P.ldc + j) = Elem<T>::pack(o);
-                        }
-                    }
-                } else {  // XMA_EPI_SWIGLU_BWD
-                    const int64_t n = n0 + cc * PV;
-                    if (n < P.n) {
-                        const T* h = reinterpret_cast<const T*>(P.aux) + p * P.ld_aux;
-                        float u[PV], g[PV], d[PV], du[PV], dg[PV];
-                        Elem<T>::unpack(*reinterpret_cast<const uint4*>(h + n), u);
-                        Elem<T>::unpack(*reinterpret_cast<const uint4*>(h + P.n + n), g);
-                        Elem<T>::unpack(chunk_at(cc), d);
+            for (int it = 0; it < IT; ++it) {
+                const int br = buffer_row(it);
+                const int64_t i = tile_i0 + tile_row(mi, br);
+                if (i < P.n && j < P.k) *reinterpret_cast<u32x4_t*>(out + i * P.ldc) = chunk_at(br, cc);
+            }
+        } else if constexpr (EPI == XMA_EPI_NONE) {
+            const int64_t n = n0 + cc * PV;
 #pragma unroll
-                        for (int q = 0; q < PV; ++q) {
-                            const float sg = sigmoid_fast(g[q]);
-                            dg[q] = d[q] * u[q] * (sg + g[q] * sg * (1.0f - sg));
-                            du[q] = d[q] * g[q] * sg;
-                        }
-                        *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = Elem<T>::pack(du);
-                        *reinterpret_cast<uint4*>(C + orow * P.ldc + P.n + n) = Elem<T>::pack(dg);
-                    }
+            for (int it = 0; it < IT; ++it)
+                if (out_row[it] >= 0 && n < P.n)
+                    *reinterpret_cast<u32x4_t*>(C + (int64_t)out_row[it] * P.ldc + n) = chunk_at(buffer_row(it), cc);
+        } else if constexpr (EPI == XMA_EPI_SWIGLU) {
+            // The slab row holds 16 chunks of the up half, then the 16 matching chunks of the gate half.  Thread
+            // cc handles chunk pair cc % 16 on every other owned row (even `it` for cc < 16, odd otherwise), so
+            // that every lane computes.
+            constexpr int HALF_CHUNKS = C_CHUNKS / 2;
+            const int64_t half_n = P.n / 2;
+            const int pair = cc % HALF_CHUNKS;
+            const int64_t j = n0 + pair * PV;
+#pragma unroll
+            for (int it2 = 0; it2 < IT / 2; ++it2) {
+                const bool odd = cc >= HALF_CHUNKS;
+                const int32_t row_out = odd ? out_row[2 * it2 + 1] : out_row[2 * it2];
+                const int br = tid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
+                if (row_out < 0 || j >= half_n) continue;
+                const int64_t p = m_begin + tile_row(mi, br);
+                const u32x4_t up = chunk_at(br, pair), gate = chunk_at(br, pair + HALF_CHUNKS);
+                if (P.aux) {
+                    T* h = reinterpret_cast<T*>(P.aux) + p * P.ld_aux;
+                    *reinterpret_cast<u32x4_t*>(h + j) = up;
+                    *reinterpret_cast<u32x4_t*>(h + half_n + j) = gate;
                 }
+                float u[PV], g[PV], o[PV];
+                Elem<T>::unpack(to_uint4(up), u);
+                Elem<T>::unpack(to_uint4(gate), g);
+#pragma unroll
+                for (int q = 0; q < PV; ++q) o[q] = u[q] * (g[q] * sigmoid_fast(g[q]));
+                *reinterpret_cast<uint4*>(C + (int64_t)row_out * P.ldc + j) = Elem<T>::pack(o);
+            }
+        } else {  // XMA_EPI_SWIGLU_BWD
+            const int64_t n = n0 + cc * PV;
+            if constexpr (mi + 1 < MI) load_saved(mi + 1, hu[(mi + 1) & 1], hg[(mi + 1) & 1], orow[mi + 1 < MI ? mi + 1 : 0]);
+#pragma unroll
+            for (int it = 0; it < IT; ++it) {
+                if (out_row[it] < 0 || n >= P.n) continue;
+                float u[PV], g[PV], d[PV], du[PV], dg[PV];
+                Elem<T>::unpack(to_uint4(hu[mi & 1][it]), u);
+                Elem<T>::unpack(to_uint4(hg[mi & 1][it]), g);
+                Elem<T>::unpack(to_uint4(chunk_at(buffer_row(it), cc)), d);
+#pragma unroll
+                for (int q = 0; q < PV; ++q) {
+                    const float sg = sigmoid_fast(g[q]);
+                    const float t = g[q] * sg;
+                    du[q] = d[q] * t;
+                    dg[q] = d[q] * u[q] * (sg + t * (1.0f - sg));
+                }
+                T* out = C + (int64_t)out_row[it] * P.ldc;
+                *reinterpret_cast<uint4*>(out + n) = Elem<T>::pack(du);
+                *reinterpret_cast<uint4*>(out + P.n + n) = Elem<T>::pack(dg);
             }
         }
     };
-    store_rows(slab<0>(), 0);
-    store_rows(slab<1>(), 1);
-    store_rows(slab<2>(), 2);
-    store_rows(slab<3>(), 3);
+    store_rows(slab<0>(), std::integral_constant<int, 0>{}, orow[0]);
+    store_rows(slab<1>(), std::integral_constant<int, 1>{}, orow[1]);
+    store_rows(slab<2>(), std::integral_constant<int, 2>{}, orow[2]);
+    store_rows(slab<3>(), std::integral_constant<int, 3>{}, orow[3]);
 }
 
 template <typename T, int KIND, int EPI, typename Pipe>
@@ -507,16 +709,18 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
 
 template <typename T>
 static int dispatch(const xma_grouped_gemm_args& a, hipStream_t stream) {
-    using Pipe = Pipe32x4;
+    using PipeTN = XMA_PIPE_TN;
+    using PipeNN = XMA_PIPE_NN;
+    using PipeMT = XMA_PIPE_MT;
     switch (a.kind) {
         case XMA_GEMM_TN:
-            if (a.epilogue == XMA_EPI_SWIGLU) return launch<T, XMA_GEMM_TN, XMA_EPI_SWIGLU, Pipe>(a, stream);
-            return launch<T, XMA_GEMM_TN, XMA_EPI_NONE, Pipe>(a, stream);
+            if (a.epilogue == XMA_EPI_SWIGLU) return launch<T, XMA_GEMM_TN, XMA_EPI_SWIGLU, PipeTN>(a, stream);
+            return launch<T, XMA_GEMM_TN, XMA_EPI_NONE, PipeTN>(a, stream);
         case XMA_GEMM_NN:
-            if (a.epilogue == XMA_EPI_SWIGLU_BWD) return launch<T, XMA_GEMM_NN, XMA_EPI_SWIGLU_BWD, Pipe>(a, stream);
-            return launch<T, XMA_GEMM_NN, XMA_EPI_NONE, Pipe>(a, stream);
+            if (a.epilogue == XMA_EPI_SWIGLU_BWD) return launch<T, XMA_GEMM_NN, XMA_EPI_SWIGLU_BWD, PipeNN>(a, stream);
+            return launch<T, XMA_GEMM_NN, XMA_EPI_NONE, PipeNN>(a, stream);
         default:
-            return launch<T, XMA_GEMM_MT, XMA_EPI_NONE, Pipe>(a, stream);
+            return launch<T, XMA_GEMM_MT, XMA_EPI_NONE, PipeMT>(a, stream);
     }
 }
 
