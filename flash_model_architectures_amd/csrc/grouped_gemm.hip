@@ -478,7 +478,7 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
         P.col_tiles = (int32_t)ceil_div(n_out, bn_out);
         grid = grid_for_tiles(rt, P.col_tiles);
         hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(1024), 0, stream, a.expert_offsets, a.num_experts,
-                           Cfg::BM, ws + 4, ws + 4 + rt, ws);
+                           Cfg::BM, ws + 4, ws + 4 + rt, ws, nullptr);
     }
     XMA_REQUIRE(grid < ((int64_t)1 << 31), "xma_grouped_gemm: %lld tiles exceed the grid limit", (long long)grid);
     (void)PV;
@@ -549,8 +549,9 @@ extern "C" {
 int64_t xma_grouped_gemm_workspace_bytes(int32_t num_experts, int64_t rows) {
     if (num_experts < 1 || rows < 0) return -1;
     (void)largest_bm();
+    // tile tables (sized for the smallest tile height of any kernel), then the split-K counters and partials
     const int64_t rt = max_row_tiles(rows, num_experts, smallest_bm());
-    return (4 + 2 * rt) * (int64_t)sizeof(int32_t);
+    return tile_table_bytes(rt) + split_region_bytes();
 }
 
 int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {

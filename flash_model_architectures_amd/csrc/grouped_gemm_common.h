@@ -35,7 +35,21 @@ struct GemmParams {
     int32_t num_experts, in_fan_out, idx_is_i64;
     int32_t row_tiles_max;  // upper bound used for the grid (TN/NN); MT: row tiles per expert
     int32_t col_tiles;
+    // split-K of the last, partly filled round of tiles (16-bit TN/NN kernels)
+    int32_t* split_counters;  // [kSplitSlots] arrivals per split tile, zero at launch
+    float* split_partials;    // [kSplitSlots][tile] fp32 accumulators of the parts
+    int32_t num_cu;
 };
+
+// At most kSplitSlots (tile, part) pairs exist at a time: the split tiles are those of one round of the device.
+constexpr int kSplitSlots = 256;
+constexpr int kMaxSplit = 4;
+constexpr int kSplitMaxRounds = 8;
+constexpr int64_t kSplitTileFloats = 256 * 256;
+inline int64_t tile_table_bytes(int64_t row_tiles) { return ((4 + 2 * row_tiles) * (int64_t)sizeof(int32_t) + 255) / 256 * 256; }
+inline int64_t split_region_bytes() {
+    return kSplitSlots * (int64_t)sizeof(int32_t) + kSplitSlots * kSplitTileFloats * (int64_t)sizeof(float);
+}
 
 // routed row p -> source row of the gathered operand (indices are < 2^31, so divide in 32 bits)
 __device__ __forceinline__ int64_t source_row(const GemmParams& P, int64_t p) {
@@ -46,8 +60,10 @@ __device__ __forceinline__ int64_t source_row(const GemmParams& P, int64_t p) {
 static __global__ __launch_bounds__(1024) void build_row_tiles_kernel(const int32_t* __restrict__ offsets, int E, int BM,
                                                                 int32_t* __restrict__ tile_expert,
                                                                 int32_t* __restrict__ tile_row0,
-                                                                int32_t* __restrict__ tile_count) {
+                                                                int32_t* __restrict__ tile_count,
+                                                                int32_t* __restrict__ split_counters) {
     __shared__ int32_t part[1024];
+    if (split_counters != nullptr && threadIdx.x < kSplitSlots) split_counters[threadIdx.x] = 0;
     const int per = (E + 1023) / 1024;
     const int e0 = threadIdx.x * per;
     int32_t s = 0;
@@ -113,6 +129,58 @@ __device__ __forceinline__ bool locate_tile(int row_tiles, int col_tiles, int& r
     col_tile = in_band / band_rows;
     return col_tile < col_tiles;
 }
+
+// Row-grouped kinds with split-K of the remainder.  With T tiles on a device of C compute units the first
+// floor(T / C) * C tiles fill whole rounds; the R = T mod C tiles of the last round would leave C - R units idle
+// for a whole tile time, so each of them is cut along the reduction into S = min(kMaxSplit, C / R, stages)
+// parts that run side by side.  (Only when the launch has fewer than kSplitMaxRounds rounds: the idle units of
+// a last round matter less the more rounds there are, and the parts cost a reduction.)  Work-groups are dealt per XCD as in locate_tile<false>: XCD x takes the x-th
+// eighth of the whole tiles, then the x-th eighth of the parts (part-major, so neighbours share panels).
+struct TileWork {
+    int row_tile, col_tile;
+    int part, parts;  // this work-group reduces stages [part * n / parts, (part + 1) * n / parts)
+    int split_tile;   // index of the tile among the split ones
+    int split_tiles;
+};
+__device__ __forceinline__ bool locate_work(int row_tiles, int col_tiles, int num_cu, int64_t stages, TileWork& w) {
+    const int xcd = blockIdx.x % kNumXcd;
+    const int local = blockIdx.x / kNumXcd;
+    const int total = row_tiles * col_tiles;
+    const int whole = total / num_cu * num_cu;  // num_cu is a multiple of kNumXcd
+    const int rem = total - whole;
+    int parts = rem > 0 && total < kSplitMaxRounds * num_cu ? num_cu / rem : 1;
+    parts = parts > kMaxSplit ? kMaxSplit : parts;
+    parts = parts > stages ? (int)stages : parts;
+    parts = parts < 1 ? 1 : parts;
+    const int whole_per_xcd = whole / kNumXcd;
+    int tile;
+    if (local < whole_per_xcd) {
+        tile = xcd * whole_per_xcd + local;
+        w.part = 0;
+        w.parts = 1;
+        w.split_tile = 0;
+    } else {
+        const int items = rem * parts;
+        const int per_xcd = (items + kNumXcd - 1) / kNumXcd;
+        const int l = local - whole_per_xcd;
+        const int q = xcd * per_xcd + l;
+        if (l >= per_xcd || q >= items) return false;
+        w.part = q / rem;
+        w.split_tile = q - w.part * rem;
+        w.parts = parts;
+        tile = whole + w.split_tile;
+    }
+    w.split_tiles = rem;
+    const int per_band = kBandTiles * col_tiles;
+    const int band = tile / per_band, in_band = tile - band * per_band;
+    const int band_first = band * kBandTiles;
+    const int band_rows = row_tiles - band_first < kBandTiles ? row_tiles - band_first : kBandTiles;
+    w.row_tile = band_first + in_band % band_rows;
+    w.col_tile = in_band / band_rows;
+    return true;
+}
+// number of work-groups that covers every case of locate_work() for up to `tiles` tiles
+inline int64_t grid_for_work(int64_t tiles) { return (ceil_div(tiles, kNumXcd) + kSplitSlots / kNumXcd + 1) * kNumXcd; }
 
 // number of work-groups that covers up to `row_tiles` x `col_tiles` under either dealing of locate_tile()
 inline int64_t grid_for_tiles(int64_t row_tiles, int64_t col_tiles) {

@@ -225,6 +225,12 @@ struct OperandLoads {
         wave_lds = wave * 1024;
     }
 
+    // Make stage 0 the stage `first` of the reduction (split-K parts start in the middle).
+    __device__ __forceinline__ void skip_stages(int64_t first) {
+#pragma unroll
+        for (int i = 0; i < (PLAN == PLAN_ROWS ? LOADS : 1); ++i) ptr[i] += first * step;
+    }
+
     // Issue this wave's loads I0 <= i < I1 of the stage `stage` into the tile at slab_base + tile_off.
     template <int I0, int I1>
     __device__ __forceinline__ void issue(char* slab_base, int tile_off, int64_t stage, int64_t red_len) const {
@@ -465,9 +471,16 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     k.lane = tid & 63;
     k.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    const int row_tiles = KIND == XMA_GEMM_MT ? P.row_tiles_max * P.num_experts : P.tile_count[0];
     int row_tile, col_tile;
-    if (!locate_tile<XMA_SPREAD(KIND)>(row_tiles, P.col_tiles, row_tile, col_tile)) return;
+    TileWork work;
+    work.parts = 1;
+    if constexpr (KIND == XMA_GEMM_MT) {
+        if (!locate_tile<true>(P.row_tiles_max * P.num_experts, P.col_tiles, row_tile, col_tile)) return;
+    } else {
+        if (!locate_work(P.tile_count[0], P.col_tiles, P.num_cu, (P.k + K::BK - 1) / K::BK, work)) return;
+        row_tile = work.row_tile;
+        col_tile = work.col_tile;
+    }
 
     const T* A = reinterpret_cast<const T*>(P.a);
     const T* B = reinterpret_cast<const T*>(P.b);
@@ -515,6 +528,15 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             k.lb.setup_strided(k.wave, k.lane, W + n0, P.ldb, P.n - n0);
         }
     }
+    if constexpr (KIND != XMA_GEMM_MT) {
+        if (work.parts > 1) {
+            const int64_t stages = (k.red_len + K::BK - 1) / K::BK;
+            const int64_t first = work.part * stages / work.parts, end = (work.part + 1) * stages / work.parts;
+            k.la.skip_stages(first);
+            k.lb.skip_stages(first);
+            k.red_len = (end * K::BK < k.red_len ? end * K::BK : k.red_len) - first * K::BK;
+        }
+    }
     k.init_fragments();
 
     f32x16_t acc[MI][NI];
@@ -526,6 +548,57 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
 
     k.run(acc);
+
+    // ---- split-K: every part parks its accumulators; the part that arrives last adds them up in part order
+    // (so the result does not depend on the arrival order) and goes on to the epilogue ----
+    if constexpr (KIND != XMA_GEMM_MT) {
+        if (work.parts > 1) {
+            typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+            auto part_buffer = [&](int part) {
+                return reinterpret_cast<f32x4_t*>(P.split_partials +
+                                                  (int64_t)(part * work.split_tiles + work.split_tile) * kSplitTileFloats);
+            };
+            f32x4_t* mine = part_buffer(work.part);
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        mine[((mi * NI + ni) * 4 + g) * THREADS + tid] =
+                            f32x4_t{acc[mi][ni][4 * g], acc[mi][ni][4 * g + 1], acc[mi][ni][4 * g + 2], acc[mi][ni][4 * g + 3]};
+            __threadfence();  // this thread's partial sums are visible to the whole device ...
+            __syncthreads();  // ... and so are everybody else's, before the arrival is counted
+            int* arrivals = reinterpret_cast<int*>(slab<0>());
+            if (tid == 0)
+                arrivals[0] = __hip_atomic_fetch_add(P.split_counters + work.split_tile, 1, __ATOMIC_ACQ_REL,
+                                                     __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            const bool last = arrivals[0] == work.parts - 1;
+            __syncthreads();  // the slab is reused below
+            if (!last) return;
+            __threadfence();
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
+            for (int part = 0; part < work.parts; ++part) {
+                const f32x4_t* src = part_buffer(part);
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            const f32x4_t v = src[((mi * NI + ni) * 4 + g) * THREADS + tid];
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) acc[mi][ni][4 * g + q] += v[q];
+                        }
+            }
+        }
+    }
 
     // ---- epilogue: accumulators -> LDS (slab mi holds the 64 tile rows {wr*128 + mi*32 + 0..31}) -> HBM ----
     // Store phase: each thread owns one 16-byte chunk column (cc) and, per slab, the IT buffer rows
@@ -679,6 +752,20 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     store_rows(slab<3>(), std::integral_constant<int, 3>{}, orow[3]);
 }
 
+// Compute units of the current device, rounded down to a multiple of the XCD count and capped at the
+// number of split slots (the split-K scheme treats that many tiles as one round).
+static int compute_units() {
+    static int cached = 0;  // one device model per process
+    if (cached > 0) return cached;
+    int device = 0, count = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count < kNumXcd)
+        count = kSplitSlots;
+    count = count > kSplitSlots ? kSplitSlots : count;
+    cached = count / kNumXcd * kNumXcd;
+    return cached;
+}
+
 template <typename T, int KIND, int EPI, typename Pipe>
 static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
     GemmParams P;
@@ -695,12 +782,18 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
         P.tile_expert = ws + 4;
         P.tile_row0 = ws + 4 + rt;
         P.row_tiles_max = (int32_t)rt;
+        // the split-K region is the tail of the workspace
+        char* split = reinterpret_cast<char*>(a.workspace) +
+                      (xma_grouped_gemm_workspace_bytes(a.num_experts, a.rows) - split_region_bytes());
+        P.split_counters = reinterpret_cast<int32_t*>(split);
+        P.split_partials = reinterpret_cast<float*>(split + kSplitSlots * sizeof(int32_t));
+        P.num_cu = compute_units();
         const int bn_out = EPI == XMA_EPI_SWIGLU ? BN / 2 : BN;
         const int64_t n_out = EPI == XMA_EPI_SWIGLU ? a.n / 2 : a.n;
         P.col_tiles = (int32_t)ceil_div(n_out, bn_out);
-        grid = grid_for_tiles(rt, P.col_tiles);
+        grid = grid_for_work(rt * P.col_tiles);
         hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(1024), 0, stream, a.expert_offsets, a.num_experts, BM,
-                           ws + 4, ws + 4 + rt, ws);
+                           ws + 4, ws + 4 + rt, ws, P.split_counters);
     }
     XMA_REQUIRE(grid < ((int64_t)1 << 31), "xma_grouped_gemm: %lld tiles exceed the grid limit", (long long)grid);
     hipLaunchKernelGGL((grouped_gemm_dma_kernel<T, KIND, EPI, Pipe>), dim3((unsigned)grid), dim3(THREADS), 0, stream, P);
