@@ -5,7 +5,7 @@
  * Every entry point takes raw device pointers, sizes, strides (in elements), a dtype
  * code and a HIP stream handle passed as `void*` (a `hipStream_t`; NULL = the null
  * stream).  Nothing here allocates or frees device memory: the caller owns every
- * buffer, including the small workspaces whose sizes the `*_workspace_bytes` helpers
+ * buffer, including the workspaces whose sizes the `*_workspace_bytes` helpers
  * return.  All launches are asynchronous on the given stream.  Return value: 0 on
  * success, non-zero on a rejected argument or a failed launch; `xma_last_error()`
  * then returns a thread-local, NUL-terminated description.
@@ -182,6 +182,9 @@ int xma_swiglu_backward(const void* gate, int64_t ld_gate, const void* up, int64
  * for them (the reference pre-zeroes DW, xma/layers/moe/triton_implementation/__init__.py:121).
  * Replaces scatter2scatter (scatter_kernel.py:137-183) and group_bwd_W
  * (group_backward_kernel.py:102-125).
+ * The workspace (TN/NN) holds the row-tile tables and a fixed 64 MiB region for the fp32
+ * partial sums of tiles whose reduction is split; launches that may run concurrently need
+ * a workspace each.  The kernel initialises what it uses.
  */
 int64_t xma_grouped_gemm_workspace_bytes(int32_t num_experts, int64_t rows);
 int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream);
