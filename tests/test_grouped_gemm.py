@@ -156,3 +156,33 @@ def test_ragged_tail_rows_are_not_touched():
     ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, off, out, 1, True, True)
     ref = torch.cat([x[:1].float() @ w[0].float().T, x[1:].float() @ w[2].float().T])
     assert_close(out, ref, TOL[torch.bfloat16])
+
+
+@pytest.mark.parametrize("layout", ["TN", "NN"])
+def test_whole_rounds_plus_split_remainder(layout):
+    """More tiles than compute units, with a remainder: the first tiles run whole, the tiles of the last,
+    partly filled round are reduced in parts and summed by the part that finishes last.  Checked against fp32
+    matmuls on the device; run twice to see that the result does not depend on the arrival order."""
+
+    dev = "cuda"
+    E, K, N = 4, 320, 1792  # 7 column tiles; ~43 row tiles -> ~300 tiles on 256 compute units
+    sizes = [2700, 1, 3100, 4300]
+    M = sum(sizes)
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(E, N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)  # [E, N, K]
+    off = torch.tensor([0] + list(torch.tensor(sizes).cumsum(0)), dtype=torch.int32, device=dev)
+    idx = torch.arange(M, dtype=torch.int32, device=dev)
+    se = torch.repeat_interleave(torch.arange(E), torch.tensor(sizes)).int().to(dev)
+    if layout == "TN":
+        weights = w.permute(0, 2, 1)  # logical [E, K, N], K contiguous
+    else:
+        weights = w.permute(0, 2, 1).contiguous()  # [E, K, N], N contiguous
+    outs = []
+    for _ in range(2):
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        ops.scatter2scatter(a, weights, se, idx, off, out, 1, True, True)
+        outs.append(out)
+    ref = torch.cat([a[off[e] : off[e + 1]].float() @ w[e].float().T for e in range(E)])
+    assert_close(outs[0], ref, TOL[torch.bfloat16])
+    assert torch.equal(outs[0], outs[1])
