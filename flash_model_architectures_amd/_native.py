@@ -89,6 +89,14 @@ PROTOTYPES: dict[str, tuple] = {
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int32, c_int64, c_int, c_void_p],
     ),
+    "xma_add_expert_bias": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int, c_void_p],
+    ),
+    "xma_expert_colsum": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int32, c_int64, c_void_p, c_int64, c_int, c_void_p],
+    ),
     "xma_swiglu_forward": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p],

@@ -22,8 +22,10 @@ from ..accelerator import KernelBackend, resolve_backend
 from ..functional.routing import route_tokens, topk_softmax
 from ..functional.swiglu_packed import swiglu_packed
 from ..ops import (
+    add_expert_bias,
     combine_topk,
     down_projection_dgrad_swiglu,
+    expert_colsum,
     gate_grad,
     group,
     group_bwd_W,
@@ -48,6 +50,7 @@ class _ScatteredExperts(torch.autograd.Function):
         gates,
         grouped_in,
         grouped_out,
+        bias,
     ):
         M = sorted_expert_idxs.size(0)
         expanded = torch.empty(M, expert_weights.size(-1), device=x.device, dtype=x.dtype)
@@ -62,6 +65,14 @@ class _ScatteredExperts(torch.autograd.Function):
             x_grouped=grouped_in,
             y_grouped=grouped_out,
         )
+        if bias is not None:
+            # F.linear(x, W[e], bias[e]) of the reference's torch path (xma/layers/moe/__init__.py:103-106)
+            add_expert_bias(
+                y=expanded,
+                bias=bias,
+                sorted_expert_idxs=sorted_expert_idxs,
+                out_index=None if grouped_out else sorted_scattered_idxs,
+            )
         if gates is None:
             output, saved_expanded = expanded, None
         else:
@@ -73,6 +84,7 @@ class _ScatteredExperts(torch.autograd.Function):
             x, expert_weights, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, saved_expanded
         )
         ctx.k, ctx.grouped_in, ctx.grouped_out = k, grouped_in, grouped_out
+        ctx.has_bias = bias is not None
         return output
 
     @staticmethod
@@ -102,6 +114,11 @@ class _ScatteredExperts(torch.autograd.Function):
                 coeff=None if gates is None else gates.flatten(),
                 fan_out=1 if gates is None else gates.size(1),
             )
+
+        d_bias = None
+        if ctx.has_bias and ctx.needs_input_grad[9]:
+            d_bias = torch.empty(E, N, device=x.device, dtype=x.dtype)
+            expert_colsum(src=grouped_grad, expert_offsets=expert_offsets, out=d_bias)
 
         # weight gradient; the token gather of the up-projection is fused into the kernel
         d_weights = torch.empty_like(W)  # keeps the strides of the view
@@ -134,7 +151,7 @@ class _ScatteredExperts(torch.autograd.Function):
             d_input = torch.empty_like(x, memory_format=torch.contiguous_format)
             combine_topk(expanded=d_expanded_input, out=d_input, k=k, gates=None)
 
-        return d_input, d_weights, None, None, None, None, d_gates, None, None
+        return d_input, d_weights, None, None, None, None, d_gates, None, None, d_bias
 
 
 def scattered_experts(
@@ -147,7 +164,11 @@ def scattered_experts(
     gates: torch.Tensor | None = None,
     grouped_in: bool = False,
     grouped_out: bool = False,
+    bias: torch.Tensor | None = None,
 ) -> torch.Tensor:
+    """Same call as the reference's `scattered_experts` (triton_implementation/__init__.py:164-185) plus an
+    optional per-expert bias [E, out_features], which the reference offers on its torch path only."""
+
     return _ScatteredExperts.apply(
         inputs,
         expert_weights,
@@ -158,6 +179,7 @@ def scattered_experts(
         gates,
         grouped_in,
         grouped_out,
+        bias,
     )
 
 
@@ -285,7 +307,6 @@ class Experts(XMAModule):
         grouped_in: bool = False,
         grouped_out: bool = False,
     ) -> torch.Tensor:
-        assert self.bias is None, "the kernel path has no bias support"
         return scattered_experts(
             inputs=input,
             expert_weights=self.weight.permute(0, 2, 1),
@@ -296,6 +317,7 @@ class Experts(XMAModule):
             gates=gates,
             grouped_in=grouped_in,
             grouped_out=grouped_out,
+            bias=self.bias,
         )
 
     def extra_repr(self) -> str:
@@ -379,11 +401,12 @@ class MoE(XMAModule):
         kernel_backend: KernelBackend | None = None,
     ) -> torch.Tensor:
         resolve_backend(kernel_backend, "MoE")
-        assert self.c_fc.bias is None and self.c_proj.bias is None, "the kernel path has no bias support"
 
         routing = route_tokens(selected_experts, self.num_experts)
 
-        if self.act is swiglu_packed and self.is_glu:
+        # biases (torch path only in the reference, xma/layers/moe/__init__.py:54,79,104) go through the general
+        # pipeline, where they are added after each projection
+        if self.act is swiglu_packed and self.is_glu and self.c_fc.bias is None and self.c_proj.bias is None:
             return _SwigluExperts.apply(
                 hidden_states,
                 self.c_fc.weight,

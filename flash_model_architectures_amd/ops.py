@@ -269,6 +269,62 @@ def gate_grad(expanded: torch.Tensor, grad_out: torch.Tensor, d_gates: torch.Ten
     )
 
 
+@xma_op(mutates_args={"y"})
+def add_expert_bias(
+    y: torch.Tensor, bias: torch.Tensor, sorted_expert_idxs: torch.Tensor, out_index: torch.Tensor | None = None
+) -> None:
+    """y[r] += bias[sorted_expert_idxs[p]] for every routed row p; r = out_index[p], or p for grouped rows."""
+
+    nat.require_device(y, bias, sorted_expert_idxs)
+    assert y.dim() == 2 and bias.dim() == 2 and y.size(1) == bias.size(1) and y.dtype == bias.dtype
+    assert y.stride(1) == 1 and bias.stride(1) == 1
+    assert sorted_expert_idxs.is_contiguous() and sorted_expert_idxs.dtype in (torch.int32, torch.int64)
+    rows = sorted_expert_idxs.numel()
+    if out_index is not None:
+        assert out_index.is_contiguous() and out_index.numel() == rows and out_index.dtype in (torch.int32, torch.int64)
+    assert y.size(0) >= rows
+    nat.call(
+        "xma_add_expert_bias",
+        y.data_ptr(),
+        _row_stride(y),
+        bias.data_ptr(),
+        _row_stride(bias),
+        sorted_expert_idxs.data_ptr(),
+        int(sorted_expert_idxs.dtype == torch.int64),
+        0 if out_index is None else out_index.data_ptr(),
+        int(out_index is not None and out_index.dtype == torch.int64),
+        rows,
+        y.size(1),
+        nat.dtype_code(y),
+        nat.stream(),
+        nbytes=2 * rows * y.size(1) * y.element_size(),
+    )
+
+
+@xma_op(mutates_args={"out"})
+def expert_colsum(src: torch.Tensor, expert_offsets: torch.Tensor, out: torch.Tensor) -> None:
+    """out[e] = sum of the grouped rows of expert e of `src` (fp32 accumulation, fixed order)."""
+
+    nat.require_device(src, expert_offsets, out)
+    E = out.size(0)
+    assert src.dim() == 2 and out.dim() == 2 and src.size(1) == out.size(1) and src.dtype == out.dtype
+    assert src.stride(1) == 1 and out.stride(1) == 1
+    assert expert_offsets.dtype == torch.int32 and expert_offsets.is_contiguous() and expert_offsets.numel() == E + 1
+    nat.call(
+        "xma_expert_colsum",
+        src.data_ptr(),
+        _row_stride(src),
+        expert_offsets.data_ptr(),
+        E,
+        src.size(1),
+        out.data_ptr(),
+        _row_stride(out),
+        nat.dtype_code(src),
+        nat.stream(),
+        nbytes=(src.numel() + out.numel()) * src.element_size(),
+    )
+
+
 # ------------------------------------------------------------------------------------------------
 # swiglu
 # ------------------------------------------------------------------------------------------------

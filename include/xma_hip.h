@@ -177,6 +177,24 @@ int xma_swiglu_backward(const void* gate, int64_t ld_gate, const void* up, int64
                         int64_t ld_dup, int64_t rows, int64_t cols, int dtype, void* stream);
 
 /*
+ * Per-expert bias of a projection: y[r, :] += bias[expert_of_row[p], :] for every routed row p, where
+ * r = out_index[p] (the row's place in a scattered buffer) or p when out_index is NULL.  In place.
+ * Replaces the bias operand of F.linear on the reference's torch path
+ * (xma/layers/moe/__init__.py:103-106); the reference's kernel path has no bias (:54,79).
+ */
+int xma_add_expert_bias(void* y, int64_t ld_y, const void* bias, int64_t ld_bias, const void* expert_of_row,
+                        int expert_is_i64, const void* out_index, int idx_is_i64, int64_t rows, int64_t cols,
+                        int dtype, void* stream);
+
+/*
+ * Bias gradient: out[e, :] = sum over the grouped rows expert_offsets[e] .. expert_offsets[e+1]-1 of src,
+ * accumulated in fp32 in a fixed order.  expert_offsets: int32[num_experts + 1].  Replaces autograd's
+ * reduction for the bias of F.linear on the reference's torch path (same lines).
+ */
+int xma_expert_colsum(const void* src, int64_t ld, const int32_t* expert_offsets, int32_t num_experts,
+                      int64_t cols, void* out, int64_t ld_out, int dtype, void* stream);
+
+/*
  * Ragged batched GEMM over the experts' row groups with fp32 accumulation; see the enums
  * above for layouts and fused epilogues.  Empty groups are legal; XMA_GEMM_MT writes zeros
  * for them (the reference pre-zeroes DW, xma/layers/moe/triton_implementation/__init__.py:121).

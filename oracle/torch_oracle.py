@@ -100,12 +100,14 @@ def swiglu_backward(gate: torch.Tensor, up: torch.Tensor, dy: torch.Tensor) -> t
 # --------------------------------------------------------------------------------------------------
 # experts
 # --------------------------------------------------------------------------------------------------
-def experts_forward(grouped: torch.Tensor | list, weight: torch.Tensor, expert_frequency, return_list: bool):
-    """`Experts.torch_forward`, xma/layers/moe/__init__.py:95-111 (bias-free)."""
+def experts_forward(
+    grouped: torch.Tensor | list, weight: torch.Tensor, expert_frequency, return_list: bool, bias: torch.Tensor | None = None
+):
+    """`Experts.torch_forward`, xma/layers/moe/__init__.py:95-111."""
 
     if isinstance(grouped, torch.Tensor):
         grouped = grouped.split(expert_frequency.tolist(), dim=0)
-    out = [F.linear(grouped[e], weight[e]) for e in range(weight.size(0))]
+    out = [F.linear(grouped[e], weight[e], None if bias is None else bias[e]) for e in range(weight.size(0))]  # :103-106
     return out if return_list else torch.cat(out, dim=0)
 
 
@@ -116,6 +118,8 @@ def moe_experts(
     router_weights: torch.Tensor,
     selected_experts: torch.Tensor,
     activation: Callable = swiglu_packed,
+    b_up: torch.Tensor | None = None,
+    b_down: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """The torch branch of `MoE._compute_experts`, xma/layers/moe/__init__.py:218-219,243-262."""
 
@@ -125,9 +129,9 @@ def moe_experts(
     fan_in_index = routing.sorted_scattered_idxs // top_k  # :245
     batch_gates = router_weights.flatten()[routing.sorted_scattered_idxs]  # :248-249
     h = x[fan_in_index]  # :251
-    h = experts_forward(h, w_up, routing.expert_frequency, return_list=True)  # :253
+    h = experts_forward(h, w_up, routing.expert_frequency, return_list=True, bias=b_up)  # :253
     h = [activation(i) for i in h]  # :257
-    h = experts_forward(h, w_down, None, return_list=False)  # :258
+    h = experts_forward(h, w_down, None, return_list=False, bias=b_down)  # :258
     h = h * batch_gates.unsqueeze(-1)  # :260
     zeros = torch.zeros((x.size(0), x.size(1)), dtype=h.dtype, device=h.device)
     return zeros.index_add(0, fan_in_index, h)  # :261-262
@@ -141,6 +145,8 @@ def moe_forward(
     top_k: int,
     activation: Callable = swiglu_packed,
     logits_bias: torch.Tensor | None = None,
+    b_up: torch.Tensor | None = None,
+    b_down: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """`MoE.forward`, xma/layers/moe/__init__.py:168-203: returns (output, router_logits)."""
 
@@ -150,7 +156,7 @@ def moe_forward(
     if logits_bias is not None:
         router_logits = router_logits + logits_bias
     weights, selected = routing_weights(router_logits, top_k)
-    y = moe_experts(x2, w_up, w_down, weights, selected, activation)
+    y = moe_experts(x2, w_up, w_down, weights, selected, activation, b_up, b_down)
     return y.view(shape), router_logits
 
 

@@ -211,3 +211,51 @@ def test_mixtral_shaped_full_size_sampled():
     assert _device_rel_err(moe.c_fc.weight.grad, w_up.grad.to(dev)) <= tol
     assert _device_rel_err(moe.c_proj.weight.grad, w_down.grad.to(dev)) <= tol
     assert bool(torch.isfinite(y).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("activation", ["swiglu", "glu", "gelu"])
+def test_expert_biases(activation, dtype):
+    """`add_bias=True`: F.linear(x, W[e], bias[e]) in both projections (the reference's torch path,
+    xma/layers/moe/__init__.py:103-106), forward and every gradient including the biases'."""
+
+    T, H, I, E, k = 777, 256, 384, 6, 2
+    is_glu = activation != "gelu"
+    act_gpu = {"swiglu": xma.swiglu_packed, "glu": nn.GLU(), "gelu": nn.GELU(approximate="tanh")}[activation]
+    act_cpu = {"swiglu": to.swiglu_packed, "glu": nn.GLU(), "gelu": nn.GELU(approximate="tanh")}[activation]
+    x, w_gate, w_up, w_down, d_y = make_moe_inputs(T, H, I, E, seed=4, dtype=dtype)
+    if not is_glu:
+        w_up = w_up[:, :I].contiguous()
+    g = torch.Generator().manual_seed(9)
+    b_up = (0.3 * torch.randn(E, w_up.size(1), generator=g)).to(dtype)
+    b_down = (0.3 * torch.randn(E, H, generator=g)).to(dtype)
+
+    moe = xma.MoE(E, k, H, I, act_gpu, is_glu, True, 0.02)
+    assert moe.c_fc.bias.shape == b_up.shape and moe.c_proj.bias.shape == b_down.shape
+    with torch.no_grad():
+        moe.gate.weight.copy_(w_gate)
+        moe.c_fc.weight.copy_(w_up)
+        moe.c_proj.weight.copy_(w_down)
+        moe.c_fc.bias.copy_(b_up)
+        moe.c_proj.bias.copy_(b_down)
+    moe = moe.to(dtype).cuda()
+
+    xd = x.cuda().requires_grad_()
+    y, logits = moe(xd)
+    _, want_selected = to.routing_weights(logits.detach().cpu(), k)
+
+    f = torch.float32
+    xo, go, uo, do, bu, bd = (t.to(f).clone().requires_grad_() for t in (x, w_gate, w_up, w_down, b_up, b_down))
+    lo = F.linear(xo, go)
+    weights = F.softmax(lo.gather(1, want_selected).float(), dim=-1)
+    yo = to.moe_experts(xo, uo, do, weights, want_selected, act_cpu, bu, bd)
+    tol = TOL[dtype]
+    assert_close(y, yo, tol, "output")
+    y.backward(d_y.cuda())
+    yo.backward(d_y.to(f))
+    assert_close(xd.grad, xo.grad, tol, "dX")
+    assert_close(moe.c_fc.weight.grad, uo.grad, tol, "dW up")
+    assert_close(moe.c_proj.weight.grad, do.grad, tol, "dW down")
+    assert_close(moe.c_fc.bias.grad, bu.grad, tol, "d bias up")
+    assert_close(moe.c_proj.bias.grad, bd.grad, tol, "d bias down")
+    assert_close(moe.gate.weight.grad, go.grad, 5 * tol, "dW gate")

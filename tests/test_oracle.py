@@ -222,6 +222,39 @@ def test_moe_empty_experts_and_all_tokens_on_one():
     assert np.abs(y.numpy() - yc).max() / np.abs(yc).max() < 1e-5
 
 
+def test_moe_biases_tokenwise_and_closed_form_gradient():
+    """Biases (torch path of the reference only): a token-by-token restatement in float64 pins the forward,
+    and the bias gradients have closed forms: d b_down[e] = sum of gate * grad_out over the (token, slot)
+    pairs routed to e; with zero weights the up bias alone drives the activation."""
+
+    x, w_gate, w_up, w_down, k = _tiny(E=5, k=2, seed=6)
+    E, I2, H = w_up.shape
+    g = torch.Generator().manual_seed(2)
+    b_up, b_down = torch.randn(E, I2, generator=g), torch.randn(E, H, generator=g)
+    logits = x @ w_gate.T
+    w, idx = to.routing_weights(logits, k)
+    bu, bd = b_up.clone().requires_grad_(), b_down.clone().requires_grad_()
+    y = to.moe_experts(x, w_up, w_down, w, idx, b_up=bu, b_down=bd)
+    want = torch.zeros(x.shape, dtype=torch.float64)
+    for t in range(x.size(0)):
+        for j in range(k):
+            e = int(idx[t, j])
+            h = w_up[e].double() @ x[t].double() + b_up[e].double()
+            a = h[: I2 // 2] * F.silu(h[I2 // 2 :])
+            want[t] += w[t, j].double() * (w_down[e].double() @ a + b_down[e].double())
+    assert max_rel_err(y, want.float()) < 1e-5
+    go = torch.randn(y.shape, generator=g)
+    y.backward(go)
+    d_bd = torch.zeros(E, H, dtype=torch.float64)
+    for t in range(x.size(0)):
+        for j in range(k):
+            d_bd[int(idx[t, j])] += w[t, j].double() * go[t].double()
+    assert max_rel_err(bd.grad, d_bd.float()) < 1e-5
+    # zero weights: y[t] = sum_j w[t,j] * b_down[e]  (+ nothing from the activation of a zero up bias)
+    y0 = to.moe_experts(x, torch.zeros_like(w_up), torch.zeros_like(w_down), w, idx, b_up=torch.zeros_like(b_up), b_down=b_down)
+    assert max_rel_err(y0, (w.unsqueeze(-1) * b_down[idx]).sum(1)) < 1e-5
+
+
 def test_moe_autograd_against_explicit_backward():
     x, w_gate, w_up, w_down, k = _tiny(seed=4)
     logits = x @ w_gate.T
