@@ -1,14 +1,22 @@
 """MI355X-native MoE hot path behind the XMA Python API.
 
 Exports the names a user of `xma` imports for this path: `MoE`, `continuous_count`, `swiglu`,
-`swiglu_packed`, `KernelBackend`, `Accelerator`, `xma_op`, `CustomOp`, the call counters and
+`swiglu_packed`, `pack_sequence`, `unpack_sequence`, `KernelBackend`, `Accelerator`, `xma_op`, `CustomOp`, the call counters and
 `set_seed` (xma/__init__.py:5-29).  Everything runs through lib/libxma_hip.so.
 """
 
 from .accelerator import Accelerator, KernelBackend
 from .counters import enable_counters, get_counter_value, reset_counters
 from .custom_op import CustomOp, xma_op
-from .functional import continuous_count, route_tokens, swiglu, swiglu_packed, topk_softmax
+from .functional import (
+    continuous_count,
+    pack_sequence,
+    route_tokens,
+    swiglu,
+    swiglu_packed,
+    topk_softmax,
+    unpack_sequence,
+)
 from .layers import Experts, MoE, scattered_experts
 from .utils import ceil_divide, divide_if_divisible, set_seed
 
@@ -26,6 +34,8 @@ __all__ = [
     "topk_softmax",
     "swiglu",
     "swiglu_packed",
+    "pack_sequence",
+    "unpack_sequence",
     "Experts",
     "MoE",
     "scattered_experts",

@@ -89,6 +89,14 @@ PROTOTYPES: dict[str, tuple] = {
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int32, c_int64, c_int, c_void_p],
     ),
+    "xma_pack_sequence": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p],
+    ),
+    "xma_unpack_sequence": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p],
+    ),
     "xma_add_expert_bias": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int, c_void_p],

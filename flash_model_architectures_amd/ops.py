@@ -326,6 +326,44 @@ def expert_colsum(src: torch.Tensor, expert_offsets: torch.Tensor, out: torch.Te
 
 
 # ------------------------------------------------------------------------------------------------
+# sequence packing
+# ------------------------------------------------------------------------------------------------
+@xma_op(mutates_args={"output"})
+def pack_unpack_sequence_rocm(
+    x: torch.Tensor, output: torch.Tensor, cu_seqlens: torch.Tensor, padding_side: str, pack: bool
+) -> None:
+    """Same contract as `pack_unpack_sequence_cuda`
+    (xma/functional/sequence_packing/cuda_implementation/__init__.py:11-20): pack reads the padded
+    [B, S, ...] `x` into the packed [total, ...] `output`, unpack the other way round.  Unpack also writes
+    the zeros of the padding."""
+
+    nat.require_device(x, output, cu_seqlens)
+    assert padding_side in ("left", "right")
+    assert x.is_contiguous() and output.is_contiguous() and cu_seqlens.is_contiguous() and x.dtype == output.dtype
+    assert cu_seqlens.dim() == 1 and cu_seqlens.dtype in (torch.uint32, torch.int32, torch.int64)
+    padded, packed = (x, output) if pack else (output, x)
+    B, S = padded.size(0), padded.size(1)
+    assert cu_seqlens.numel() == B + 1
+    total = packed.size(0)
+    row = packed.numel() // total if total else (padded.numel() // (B * S) if B * S else 0)
+    assert padded.numel() == B * S * row and packed.numel() == total * row, "row shapes differ"
+    nat.call(
+        "xma_pack_sequence" if pack else "xma_unpack_sequence",
+        x.data_ptr(),
+        output.data_ptr(),
+        cu_seqlens.data_ptr(),
+        int(cu_seqlens.dtype == torch.int64),
+        B,
+        S,
+        total,
+        row * x.element_size(),
+        int(padding_side == "left"),
+        nat.stream(),
+        nbytes=(total * row + output.numel()) * x.element_size(),
+    )
+
+
+# ------------------------------------------------------------------------------------------------
 # swiglu
 # ------------------------------------------------------------------------------------------------
 @xma_op(mutates_args={"y"})

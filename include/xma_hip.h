@@ -177,6 +177,22 @@ int xma_swiglu_backward(const void* gate, int64_t ld_gate, const void* up, int64
                         int64_t ld_dup, int64_t rows, int64_t cols, int dtype, void* stream);
 
 /*
+ * Sequence packing: padded x[batch, seq_len, row] -> packed out[total_tokens, row] and back.  Sequence b
+ * holds cu_seqlens[b+1] - cu_seqlens[b] tokens (uint32 / int32, or int64 when cu_is_i64), placed at the end of
+ * its padded row block when left_padding is non-zero, at the start otherwise.  Rows are moved as bytes
+ * (row_bytes = elements per token x element size).  xma_unpack_sequence writes zeros into the padding, so
+ * the output needs no prior clearing.  Tokens of a sequence longer than seq_len have no padded position:
+ * they pack as zeros and are dropped by unpack.
+ * Replaces pack_unpack_sequence_cuda (xma/functional/sequence_packing/cuda_implementation/kernel.cu:64-137,
+ * stub cuda_implementation/__init__.py:11-20) and the zero fill that precedes its unpack calls
+ * (xma/functional/sequence_packing/__init__.py:76,139).
+ */
+int xma_pack_sequence(const void* x, void* out, const void* cu_seqlens, int cu_is_i64, int64_t batch,
+                      int64_t seq_len, int64_t total_tokens, int64_t row_bytes, int left_padding, void* stream);
+int xma_unpack_sequence(const void* x, void* out, const void* cu_seqlens, int cu_is_i64, int64_t batch,
+                        int64_t seq_len, int64_t total_tokens, int64_t row_bytes, int left_padding, void* stream);
+
+/*
  * Per-expert bias of a projection: y[r, :] += bias[expert_of_row[p], :] for every routed row p, where
  * r = out_index[p] (the row's place in a scattered buffer) or p when out_index is NULL.  In place.
  * Replaces the bias operand of F.linear on the reference's torch path

@@ -216,3 +216,40 @@ def moe_experts_backward_explicit(
     d_xe[idx] = d_xe_grouped
     d_x = d_xe.view(T, k, H).sum(-2)
     return {"x": d_x, "w_up": d_w_up, "w_down": d_w_down, "gates": d_gates}
+
+
+# --------------------------------------------------------------------------------------------------
+# sequence packing
+# --------------------------------------------------------------------------------------------------
+def _packing_indices(cu_seqlens: torch.Tensor, S: int, padding_side: str) -> tuple[torch.Tensor, torch.Tensor]:
+    """(batch index, position) of every packed token, xma/functional/sequence_packing/__init__.py:24-35."""
+
+    cu = cu_seqlens.to(torch.int64)
+    seqlens = cu[1:] - cu[:-1]
+    B = seqlens.numel()
+    batch_indices = torch.arange(B).repeat_interleave(seqlens)  # :26
+    if padding_side == "left":
+        seq_indices = torch.cat([torch.arange(S - int(n), S) for n in seqlens])  # :28-30
+    elif padding_side == "right":
+        seq_indices = torch.cat([torch.arange(int(n)) for n in seqlens])  # :31-32
+    else:
+        raise ValueError(f"unexpected padding_side ({padding_side})")
+    return batch_indices, seq_indices
+
+
+def pack_sequence(x: torch.Tensor, cu_seqlens: torch.Tensor, padding_side: str = "left") -> torch.Tensor:
+    """`_PackSequence.forward_backward_torch`, xma/functional/sequence_packing/__init__.py:20-39."""
+
+    b, s = _packing_indices(cu_seqlens, x.size(1), padding_side)
+    return x[b, s]  # :37
+
+
+def unpack_sequence(
+    x: torch.Tensor, cu_seqlens: torch.Tensor, batch_size: int, sequence_length: int, padding_side: str = "left"
+) -> torch.Tensor:
+    """`_UnpackSequence.forward_backward_torch`, xma/functional/sequence_packing/__init__.py:104-126."""
+
+    b, s = _packing_indices(cu_seqlens, sequence_length, padding_side)
+    padded = torch.zeros((batch_size, sequence_length, *x.shape[1:]), dtype=x.dtype)  # :123
+    padded[b, s] = x  # :124
+    return padded

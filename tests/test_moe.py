@@ -144,9 +144,12 @@ def test_leading_dims_inference_and_top1():
     yo, _ = to.moe_forward(xo, moe.gate.weight.detach().cpu(), moe.c_fc.weight.detach().cpu(),
                            moe.c_proj.weight.detach().cpu(), 1)
     assert_close(y.reshape(10, 64), yo, 1e-5)
-    biased = xma.MoE(4, 2, 64, 32, xma.swiglu_packed, True, True, 0.02).cuda()
-    with pytest.raises(AssertionError):
-        biased(x)  # the kernel path has no bias support, as in the reference
+    # zero-initialised biases (reset_parameters, xma/layers/moe/__init__.py:122-123) change nothing
+    biased = xma.MoE(4, 1, 64, 32, xma.swiglu_packed, True, True, 0.02).cuda()
+    biased.load_state_dict({**moe.state_dict(), "c_fc.bias": biased.c_fc.bias, "c_proj.bias": biased.c_proj.bias})
+    with torch.no_grad():
+        yb, _ = biased(x)
+    assert_close(yb, y, 1e-5)
 
 
 def test_fused_and_general_pipelines_agree():
