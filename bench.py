@@ -29,11 +29,11 @@ PEAK_HBM_BYTES = 8.0e12
 # HBM-side bytes per launch of the grouped GEMM kernels at this workload, from rocprofv3 FETCH_SIZE (x 2.0) and
 # WRITE_SIZE (x 1.0), the factors a plain 1 GiB copy gives; see profiles/moe_c2_bench_rocprofv3.txt
 MEASURED_TRAFFIC_BYTES = {
-    "xma_grouped_gemm/MT": (2250731 * 2.0 + 1978368) * 1024,
-    "xma_grouped_gemm/TN+swiglu": (3883530 * 2.0 + 2122746) * 1024,
-    "xma_grouped_gemm/TN": (1858099 * 2.0 + 324476) * 1024,
-    "xma_grouped_gemm/NN+swiglu_bwd": (2422025 * 2.0 + 1298368) * 1024,
-    "xma_grouped_gemm/NN": (3646470 * 2.0 + 347398) * 1024,
+    "xma_grouped_gemm/MT": (2245838 * 2.0 + 1978368) * 1024,
+    "xma_grouped_gemm/TN+swiglu": (3856566 * 2.0 + 2122745) * 1024,
+    "xma_grouped_gemm/TN": (1857684 * 2.0 + 324492) * 1024,
+    "xma_grouped_gemm/NN+swiglu_bwd": (2421923 * 2.0 + 1298368) * 1024,
+    "xma_grouped_gemm/NN": (3646482 * 2.0 + 347394) * 1024,
 }
 
 WORKLOAD = {
