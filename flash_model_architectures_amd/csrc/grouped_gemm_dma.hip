@@ -323,6 +323,7 @@ struct Kernel {
     int64_t red_len;
     int wave, lane;
     int a_off[4], b_off[4];  // variable parts of the fragment offsets (see fragment_offsets)
+    int active_m;            // 32-row blocks of this wave's 128 tile rows that hold existing rows (wave-uniform)
     u32x4_t fa[2][MI], fb[2][NI];  // fragments: the block being multiplied and the one being read
 
     template <int P, int I0, int I1> __device__ __forceinline__ void issue_a(int64_t stage) {
@@ -354,25 +355,30 @@ struct Kernel {
         fragment_offsets<B_STRIDED, NI>((wave % WAVES_N) * WN, b_off);
     }
 
-    // Fragments of reduction block kk of the stage held at cycle position P.
-    template <int P>
+    // Fragments of reduction block kk of the stage held at cycle position P.  FULL = false: a tile whose last
+    // rows do not exist (the tail of an expert's rows) only touches this wave's first active_m 32-row blocks.
+    template <int P, bool FULL>
     __device__ __forceinline__ void read_fragments(int kk, u32x4_t (&af)[MI], u32x4_t (&bf)[NI]) const {
         using At = typename Pipe::template At<P>;
         const char* ta = slab<At::A_SLAB>();
         const char* tb = slab<At::B_SLAB>();
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
-            af[mi] = read_fragment<A_STRIDED>(ta, At::A_OFF + fragment_offset<A_STRIDED>(a_off, mi, kk));
+            if (FULL || mi < active_m)
+                af[mi] = read_fragment<A_STRIDED>(ta, At::A_OFF + fragment_offset<A_STRIDED>(a_off, mi, kk));
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni)
             bf[ni] = read_fragment<B_STRIDED>(tb, At::B_OFF + fragment_offset<B_STRIDED>(b_off, ni, kk));
     }
 
+    template <bool FULL>
     __device__ __forceinline__ void multiply(const u32x4_t (&af)[MI], const u32x4_t (&bf)[NI], f32x16_t (&acc)[MI][NI]) {
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
+            if (FULL || mi < active_m) {
 #pragma unroll
-            for (int ni = 0; ni < NI; ++ni) Mma<T>::run(bf[ni], af[mi], acc[mi][ni]);
+                for (int ni = 0; ni < NI; ++ni) Mma<T>::run(bf[ni], af[mi], acc[mi][ni]);
+            }
     }
 
     // Asks the instruction scheduler to spread the LDS reads (and, with DMA, the loads) of one phase evenly
@@ -405,43 +411,51 @@ struct Kernel {
     // branch-free: stages past the end of the reduction fetch the zero page, which keeps the count of loads
     // in flight the same at every step and lets the compiler see that the loop needs no other wait on
     // vector memory.
-    template <int P, int PH>
+    template <int P, int PH, bool FULL>
     __device__ __forceinline__ void phases_before_barrier(int64_t s, f32x16_t (&acc)[MI][NI]) {
         if constexpr (PH + 1 < Pipe::KK) {
             Pipe::template issue_phase<P, PH>(*this, s);
-            read_fragments<P>(PH + 1, fa[(PH + 1) & 1], fb[(PH + 1) & 1]);
-            multiply(fa[PH & 1], fb[PH & 1], acc);
-            interleave_phase();
-            phases_before_barrier<P, PH + 1>(s, acc);
+            read_fragments<P, FULL>(PH + 1, fa[(PH + 1) & 1], fb[(PH + 1) & 1]);
+            multiply<FULL>(fa[PH & 1], fb[PH & 1], acc);
+            if constexpr (FULL) interleave_phase();
+            phases_before_barrier<P, PH + 1, FULL>(s, acc);
         }
     }
-    template <int P>
+    template <int P, bool FULL>
     __device__ __forceinline__ void step(int64_t s, f32x16_t (&acc)[MI][NI]) {
         constexpr int KK = Pipe::KK;
-        phases_before_barrier<P, 0>(s, acc);
+        phases_before_barrier<P, 0, FULL>(s, acc);
         wait_vmcnt_and_lds<Pipe::WAIT>();
         block_barrier();
         Pipe::template issue_phase<P, KK - 1>(*this, s);
-        read_fragments<(P + 1) % Pipe::CYCLE>(0, fa[KK & 1], fb[KK & 1]);
-        multiply(fa[(KK - 1) & 1], fb[(KK - 1) & 1], acc);
-        interleave_phase();
+        read_fragments<(P + 1) % Pipe::CYCLE, FULL>(0, fa[KK & 1], fb[KK & 1]);
+        multiply<FULL>(fa[(KK - 1) & 1], fb[(KK - 1) & 1], acc);
+        if constexpr (FULL) interleave_phase();
     }
 
-    template <int P>
+    template <int P, bool FULL>
     __device__ __forceinline__ void steps_from(int64_t s, int64_t count, f32x16_t (&acc)[MI][NI]) {
         if constexpr (P < Pipe::CYCLE) {
             if (P < count) {
-                step<P>(s + P, acc);
-                steps_from<P + 1>(s, count, acc);
+                step<P, FULL>(s + P, acc);
+                steps_from<P + 1, FULL>(s, count, acc);
             }
         }
     }
-    template <int P>
+    template <int P, bool FULL>
     __device__ __forceinline__ void full_cycle(int64_t s, f32x16_t (&acc)[MI][NI]) {
         if constexpr (P < Pipe::CYCLE) {
-            step<P>(s + P, acc);
-            full_cycle<P + 1>(s, acc);
+            step<P, FULL>(s + P, acc);
+            full_cycle<P + 1, FULL>(s, acc);
         }
+    }
+
+    template <bool FULL>
+    __device__ __forceinline__ void run_stages(int64_t num_stages, f32x16_t (&acc)[MI][NI]) {
+        read_fragments<0, FULL>(0, fa[0], fb[0]);
+        int64_t s = 0;
+        for (; s + Pipe::CYCLE <= num_stages; s += Pipe::CYCLE) full_cycle<0, FULL>(s, acc);
+        steps_from<0, FULL>(s, num_stages - s, acc);  // fewer than CYCLE steps remain
     }
 
     __device__ __forceinline__ void run(f32x16_t (&acc)[MI][NI]) {
@@ -450,11 +464,12 @@ struct Kernel {
             Pipe::prologue(*this);
             wait_vmcnt<Pipe::PROLOGUE_WAIT>();
             block_barrier();
-            read_fragments<0>(0, fa[0], fb[0]);
-            int64_t s = 0;
-            for (; s + Pipe::CYCLE <= num_stages; s += Pipe::CYCLE) full_cycle<0>(s, acc);
-            steps_from<0>(s, num_stages - s, acc);  // fewer than CYCLE steps remain
-            wait_vmcnt<0>();                         // the trailing zero-page loads
+            // The two loops issue the same loads and meet at the same barriers, so waves of one work-group may
+            // take different ones.  The row-grouped kinds take the second for the tail tile of an expert's rows:
+            // its cost then follows the rows that exist (plus the full weight panel it still has to stream).
+            if (KIND == XMA_GEMM_MT || active_m == MI) run_stages<true>(num_stages, acc);
+            else run_stages<false>(num_stages, acc);
+            wait_vmcnt<0>();  // the trailing zero-page loads
         }
         block_barrier();  // every wave is done reading the slabs; no load is in flight any more
     }
@@ -538,6 +553,12 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         }
     }
     k.init_fragments();
+    k.active_m = MI;
+    if constexpr (KIND != XMA_GEMM_MT) {
+        const int rows_here = (int)(m_end - m_begin) - (k.wave / WAVES_N) * WM;
+        const int blocks = (rows_here + 31) / 32;
+        k.active_m = __builtin_amdgcn_readfirstlane(blocks < 0 ? 0 : blocks > MI ? MI : blocks);
+    }
 
     f32x16_t acc[MI][NI];
 #pragma unroll
