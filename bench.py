@@ -7,7 +7,7 @@ throughput in tokens/s, the roofline position of the dominant kernel (timed with
 launch stream during the timed steps) and a CPU baseline: the torch restatement of the
 reference's torch path (oracle/torch_oracle.py) timed on this host's cores on a bounded sample.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-aux]
 """
 
 from __future__ import annotations
@@ -54,6 +54,7 @@ def _parse() -> argparse.Namespace:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-aux", action="store_true", help="skip the stand-alone timings of the HBM-bound kernels")
     ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
     ap.add_argument(
         "--copy-probe",
@@ -99,6 +100,65 @@ def _cpu_baseline(moe, x, d_y, sample_tokens: int) -> dict:
         f"1 timed iteration after 1 warm-up ({seconds:.2f} s); per-expert weight-gradient zero fills do not "
         "shrink with the sample, so the full-size rate is no lower than this",
     }
+
+
+def _aux_hbm_kernels(T: int, H: int, I: int, E: int, k: int) -> list:
+    """Stand-alone timings (events on the current stream, outside the timed steps) of the HBM-bound kernels of
+    the path at this workload's sizes, plus the histogram / permutation / row moves at the sizes the survey
+    names for them (2^20 ids into 256 bins, 2^20 x 4096 bf16 rows; the histogram also at 2^28 ids, which does
+    not fit the Infinity Cache)."""
+
+    import torch
+
+    import flash_model_architectures_amd as xma
+    from flash_model_architectures_amd import ops
+
+    dev, dt = "cuda", torch.bfloat16
+    out = []
+
+    def timed(name, fn, nbytes, iters=10):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(end) / iters
+        out.append(
+            {
+                "kernel": name,
+                "bytes": nbytes,
+                "avg_ms": round(ms, 4),
+                "gbps": round(nbytes / ms / 1e6, 1),
+                "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / PEAK_HBM_BYTES, 4),
+            }
+        )
+
+    M = T * k
+    h = torch.randn(M, 2 * I, device=dev, dtype=dt)
+    a = torch.empty(M, I, device=dev, dtype=dt)
+    up, gate = h.chunk(2, -1)
+    timed(f"swiglu forward [{M}, {I}]", lambda: ops.swiglu_forward_rocm(gate, up, a), 3 * M * I * 2)
+    dh = torch.empty_like(h)
+    d_up, d_gate = dh.chunk(2, -1)
+    timed(f"swiglu backward [{M}, {I}]", lambda: ops.swiglu_backward_rocm(gate, up, a, d_gate, d_up), 5 * M * I * 2)
+    del h, a, dh
+    for n in (1 << 20, 1 << 28):
+        ids = torch.randint(0, 256, (n,), dtype=torch.int32, device=dev)
+        counts = torch.empty(256, dtype=torch.uint32, device=dev)
+        timed(f"continuous_count 2^{n.bit_length() - 1} int32 ids, 256 bins", lambda: ops.continuous_count_rocm(ids, counts, 256), n * 4 + 1024)
+    ids = torch.randint(0, 256, (1 << 20,), dtype=torch.int32, device=dev)
+    timed("route_build 2^20 ids, 256 experts (count + offsets + stable permutation)", lambda: xma.route_tokens(ids, 256), 3 * (1 << 20) * 4)
+    perm = xma.route_tokens(ids, 256).sorted_scattered_idxs
+    rows = torch.empty(1 << 20, 4096, dtype=dt, device=dev).normal_()
+    moved = torch.empty_like(rows)
+    nbytes = 2 * rows.numel() * 2 + (1 << 20) * 4
+    timed("gather rows [2^20, 4096] bf16", lambda: ops.group(rows, perm, moved, None, 1), nbytes, iters=5)
+    timed("scatter rows [2^20, 4096] bf16", lambda: ops.ungroup(rows, perm, moved), nbytes, iters=5)
+    return out
 
 
 def main() -> int:
@@ -216,6 +276,8 @@ def main() -> int:
         "roofline": roofline,
         "kernels": kernels,
     }
+    if not args.no_aux:
+        result["aux_hbm_kernels"] = _aux_hbm_kernels(T, H, I, E, k)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = _cpu_baseline(moe, x, d_y, args.cpu_sample_tokens)
     print(json.dumps(result))
