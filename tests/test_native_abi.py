@@ -35,6 +35,10 @@ def test_header_declares_the_expected_entry_points():
         "xma_swiglu_forward",
         "xma_swiglu_backward",
         "xma_grouped_gemm",
+        "xma_add_expert_bias",
+        "xma_expert_colsum",
+        "xma_pack_sequence",
+        "xma_unpack_sequence",
         "xma_last_error",
     ]:
         assert required in names
@@ -79,13 +83,15 @@ def test_struct_layout_matches_header_field_order():
 
 
 def test_public_surface_mirrors_the_reference_names():
-    for name in ["MoE", "continuous_count", "swiglu", "swiglu_packed", "KernelBackend", "Accelerator", "xma_op",
-                 "CustomOp", "enable_counters", "get_counter_value", "reset_counters", "set_seed"]:
+    for name in ["MoE", "continuous_count", "swiglu", "swiglu_packed", "pack_sequence", "unpack_sequence",
+                 "KernelBackend", "Accelerator", "xma_op", "CustomOp", "enable_counters", "get_counter_value",
+                 "reset_counters", "set_seed"]:
         assert hasattr(xma, name), name
     assert [b.value for b in xma.KernelBackend] == ["cuda", "nki", "pallas", "rocm", "torch", "triton"]
     assert xma.Accelerator.get_kernel_backend() is xma.KernelBackend.rocm
     for op in ["continuous_count_rocm", "scatter2scatter", "group", "group_bwd_W", "swiglu_forward_rocm",
-               "swiglu_backward_rocm", "route_build_rocm", "topk_softmax_rocm"]:
+               "swiglu_backward_rocm", "route_build_rocm", "topk_softmax_rocm", "pack_unpack_sequence_rocm",
+               "add_expert_bias", "expert_colsum"]:
         assert hasattr(torch.ops.xma, op), f"xma::{op} is not registered"
 
 
@@ -144,3 +150,20 @@ def test_counters_and_argument_checks():
         xma.swiglu(torch.zeros(2, 4), torch.zeros(2, 5))
     with pytest.raises(AssertionError):
         xma.swiglu_packed(torch.zeros(2, 5))
+
+
+def test_product_sources_never_touch_the_oracle():
+    """The oracle is test infrastructure: nothing in the package (or the alias package) imports or opens it."""
+
+    import os
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    offenders = []
+    for package in ("flash_model_architectures_amd", "xma"):
+        for folder, _, files in os.walk(os.path.join(root, package)):
+            for name in files:
+                if name.endswith((".py", ".hip", ".h")):
+                    text = open(os.path.join(folder, name), encoding="utf-8").read()
+                    if re.search(r"\boracle\b", text):
+                        offenders.append(os.path.join(folder, name))
+    assert offenders == []
