@@ -776,14 +776,15 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 // Compute units of the current device, rounded down to a multiple of the XCD count and capped at the
 // number of split slots (the split-K scheme treats that many tiles as one round).
 static int compute_units() {
-    static int cached = 0;  // one device model per process
-    if (cached > 0) return cached;
-    int device = 0, count = 0;
-    if (hipGetDevice(&device) != hipSuccess ||
-        hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count < kNumXcd)
-        count = kSplitSlots;
-    count = count > kSplitSlots ? kSplitSlots : count;
-    cached = count / kNumXcd * kNumXcd;
+    // queried once (thread-safe initialisation of a function-local static); one device model per process
+    static const int cached = [] {
+        int device = 0, count = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count < kNumXcd)
+            count = kSplitSlots;
+        count = count > kSplitSlots ? kSplitSlots : count;
+        return count / kNumXcd * kNumXcd;
+    }();
     return cached;
 }
 
