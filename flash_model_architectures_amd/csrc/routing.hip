@@ -117,16 +117,38 @@ __global__ __launch_bounds__(1024) void unit_scan_kernel(uint32_t* __restrict__ 
     const int64_t seg = (units + 15) / 16;
     const int64_t u0 = wave * seg;
     const int64_t u1 = u0 + seg < units ? u0 + seg : units;
+    // both passes keep kScanUnroll independent loads in flight per lane: the column walk is latency-bound
+    constexpr int kScanUnroll = 8;
     uint32_t s = 0;
-    if (e < E)
-        for (int64_t u = u0; u < u1; ++u) s += unit_hist[u * E + e];
+    if (e < E) {
+        int64_t u = u0;
+        for (; u + kScanUnroll <= u1; u += kScanUnroll) {
+            uint32_t v[kScanUnroll];
+#pragma unroll
+            for (int j = 0; j < kScanUnroll; ++j) v[j] = unit_hist[(u + j) * E + e];
+#pragma unroll
+            for (int j = 0; j < kScanUnroll; ++j) s += v[j];
+        }
+        for (; u < u1; ++u) s += unit_hist[u * E + e];
+    }
     seg_sum[wave][lane] = s;
     __syncthreads();
     uint32_t base = 0;
     for (int w = 0; w < wave; ++w) base += seg_sum[w][lane];
     if (e < E) {
-        for (int64_t u = u0; u < u1; ++u) {
-            uint32_t c = unit_hist[u * E + e];
+        int64_t u = u0;
+        for (; u + kScanUnroll <= u1; u += kScanUnroll) {
+            uint32_t v[kScanUnroll];
+#pragma unroll
+            for (int j = 0; j < kScanUnroll; ++j) v[j] = unit_hist[(u + j) * E + e];
+#pragma unroll
+            for (int j = 0; j < kScanUnroll; ++j) {
+                unit_hist[(u + j) * E + e] = base;
+                base += v[j];
+            }
+        }
+        for (; u < u1; ++u) {
+            const uint32_t c = unit_hist[u * E + e];
             unit_hist[u * E + e] = base;
             base += c;
         }
