@@ -1,12 +1,12 @@
 // HBM-bound row kernels of the MoE layer on gfx950: token gather (permute) with optional
 // per-row coefficient, row scatter (unpermute), top-k weighted combine / fold, and the gate
-// gradient.  Rows are moved as 16-byte vectors; a block moves kRowsPerIter rows so
-// that several independent loads are in flight per lane before the first store.
+// gradient.  Rows are moved as 16-byte vectors, kRowsPerIter rows per block and iteration (one measured
+// fastest on 4-8 KiB rows: many small blocks keep more requests in flight than fewer, longer ones).
 #include "common.h"
 
 namespace xma {
 
-constexpr int kRowsPerIter = 2;
+constexpr int kRowsPerIter = 1;
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
