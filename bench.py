@@ -55,7 +55,7 @@ def _parse() -> argparse.Namespace:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aux", action="store_true", help="skip the stand-alone timings of the HBM-bound kernels")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
     ap.add_argument(
         "--copy-probe",
         action="store_true",
