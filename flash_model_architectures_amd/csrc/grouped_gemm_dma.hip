@@ -107,6 +107,16 @@ __device__ __forceinline__ int opaque(int v) {
     return v;
 }
 
+// The epilogue requests what it needs from HBM and LDS in batches and uses the values afterwards.  Left alone,
+// the compiler sinks each load into the conditional block that uses it and then waits for them one by one;
+// pin() makes the value live where it is called, and batch_fence() keeps the scheduler from moving the uses
+// up between the requests.
+template <typename V>
+__device__ __forceinline__ void pin(V& v) {
+    asm volatile("" : "+v"(v));
+}
+__device__ __forceinline__ void batch_fence() { __builtin_amdgcn_sched_barrier(0); }
+
 // ---- tile geometry for a stage depth of BK reduction elements ---------------------------------------
 template <int BK>
 struct Geometry {
@@ -523,12 +533,28 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         k.la.setup_strided(k.wave, k.lane, A + m_begin * P.lda + tile_i0, P.lda, P.n - tile_i0);
         k.lb.setup_strided(k.wave, k.lane, B + m_begin * P.ldb + n0, P.ldb, P.k - n0);
     } else {
-        k.la.setup_rows(k.wave, k.lane, [&](int r) -> const T* {
-            const int64_t p = m_begin + r;
-            if (p >= m_end) return nullptr;
-            const int64_t src = P.in_index ? source_row(P, p) : p;
-            return A + src * P.lda;
-        });
+        // The three ways of finding a row's source are told apart once, outside the per-row code, and rows past
+        // the end look up the tile's first row (which always exists) and are then dropped: with a branch per
+        // row the eight index loads of a lane would wait for each other.
+        auto plan_rows = [&](auto source_of) {
+            k.la.setup_rows(k.wave, k.lane, [&](int r) -> const T* {
+                const int64_t p = m_begin + r;
+                const bool exists = p < m_end;
+                const T* row = A + source_of(exists ? p : m_begin) * P.lda;
+                return exists ? row : nullptr;
+            });
+        };
+        const uint32_t fan_out = (uint32_t)P.in_fan_out;
+        if (P.in_index == nullptr)
+            plan_rows([&](int64_t p) { return p; });
+        else if (P.idx_is_i64)
+            plan_rows([&](int64_t p) {
+                return (int64_t)((uint32_t)reinterpret_cast<const int64_t*>(P.in_index)[p] / fan_out);
+            });
+        else
+            plan_rows([&](int64_t p) {
+                return (int64_t)((uint32_t)reinterpret_cast<const int32_t*>(P.in_index)[p] / fan_out);
+            });
         const T* W = B + (int64_t)expert * P.b_expert_stride;
         if constexpr (KIND == XMA_GEMM_TN) {
             if constexpr (EPI == XMA_EPI_SWIGLU) {
@@ -644,8 +670,16 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 #pragma unroll
                 for (int it = 0; it < IT; ++it) {
                     const int64_t p = m_begin + tile_row(mi, buffer_row(it));
-                    const int32_t v = index_of(p < m_end ? p : last);
-                    orow[mi][it] = p < m_end ? v : -1;
+                    orow[mi][it] = index_of(p < m_end ? p : last);
+                }
+            batch_fence();
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                for (int it = 0; it < IT; ++it) {
+                    const int64_t p = m_begin + tile_row(mi, buffer_row(it));
+                    pin(orow[mi][it]);
+                    orow[mi][it] = p < m_end ? orow[mi][it] : -1;
                 }
         };
         if (P.out_index == nullptr) fill([&](int64_t p) { return (int32_t)p; });
@@ -701,21 +735,32 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             return *reinterpret_cast<const u32x4_t*>(buf + br * (BN * 2) + ((c ^ (br & 31)) << 4));
         };
         auto to_uint4 = [](const u32x4_t& v) { return make_uint4(v[0], v[1], v[2], v[3]); };
+        // the thread's chunk of each of its IT rows of the slab, requested together
+        auto read_own_chunks = [&](u32x4_t (&v)[IT]) {
+#pragma unroll
+            for (int it = 0; it < IT; ++it) v[it] = chunk_at(buffer_row(it), cc);
+            batch_fence();
+#pragma unroll
+            for (int it = 0; it < IT; ++it) pin(v[it]);
+        };
         if constexpr (KIND == XMA_GEMM_MT) {
             const int64_t j = n0 + cc * PV;
             T* out = C + (int64_t)expert * P.c_expert_stride + j;
+            u32x4_t v[IT];
+            read_own_chunks(v);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                const int br = buffer_row(it);
-                const int64_t i = tile_i0 + tile_row(mi, br);
-                if (i < P.n && j < P.k) *reinterpret_cast<u32x4_t*>(out + i * P.ldc) = chunk_at(br, cc);
+                const int64_t i = tile_i0 + tile_row(mi, buffer_row(it));
+                if (i < P.n && j < P.k) *reinterpret_cast<u32x4_t*>(out + i * P.ldc) = v[it];
             }
         } else if constexpr (EPI == XMA_EPI_NONE) {
             const int64_t n = n0 + cc * PV;
+            u32x4_t v[IT];
+            read_own_chunks(v);
 #pragma unroll
             for (int it = 0; it < IT; ++it)
                 if (out_row[it] >= 0 && n < P.n)
-                    *reinterpret_cast<u32x4_t*>(C + (int64_t)out_row[it] * P.ldc + n) = chunk_at(buffer_row(it), cc);
+                    *reinterpret_cast<u32x4_t*>(C + (int64_t)out_row[it] * P.ldc + n) = v[it];
         } else if constexpr (EPI == XMA_EPI_SWIGLU) {
             // The slab row holds 16 chunks of the up half, then the 16 matching chunks of the gate half.  Thread
             // cc handles chunk pair cc % 16 on every other owned row (even `it` for cc < 16, odd otherwise), so
@@ -724,14 +769,27 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             const int64_t half_n = P.n / 2;
             const int pair = cc % HALF_CHUNKS;
             const int64_t j = n0 + pair * PV;
+            const bool odd = cc >= HALF_CHUNKS;
+            u32x4_t ups[IT / 2], gates[IT / 2];
 #pragma unroll
             for (int it2 = 0; it2 < IT / 2; ++it2) {
-                const bool odd = cc >= HALF_CHUNKS;
+                const int br = tid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
+                ups[it2] = chunk_at(br, pair);
+                gates[it2] = chunk_at(br, pair + HALF_CHUNKS);
+            }
+            batch_fence();
+#pragma unroll
+            for (int it2 = 0; it2 < IT / 2; ++it2) {
+                pin(ups[it2]);
+                pin(gates[it2]);
+            }
+#pragma unroll
+            for (int it2 = 0; it2 < IT / 2; ++it2) {
                 const int32_t row_out = odd ? out_row[2 * it2 + 1] : out_row[2 * it2];
                 const int br = tid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
                 if (row_out < 0 || j >= half_n) continue;
                 const int64_t p = m_begin + tile_row(mi, br);
-                const u32x4_t up = chunk_at(br, pair), gate = chunk_at(br, pair + HALF_CHUNKS);
+                const u32x4_t up = ups[it2], gate = gates[it2];
                 if (P.aux) {
                     T* h = reinterpret_cast<T*>(P.aux) + p * P.ld_aux;
                     *reinterpret_cast<u32x4_t*>(h + j) = up;
@@ -747,13 +805,15 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         } else {  // XMA_EPI_SWIGLU_BWD
             const int64_t n = n0 + cc * PV;
             if constexpr (mi + 1 < MI) load_saved(mi + 1, hu[(mi + 1) & 1], hg[(mi + 1) & 1], orow[mi + 1 < MI ? mi + 1 : 0]);
+            u32x4_t dv[IT];
+            read_own_chunks(dv);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
                 if (out_row[it] < 0 || n >= P.n) continue;
                 float u[PV], g[PV], d[PV], du[PV], dg[PV];
                 Elem<T>::unpack(to_uint4(hu[mi & 1][it]), u);
                 Elem<T>::unpack(to_uint4(hg[mi & 1][it]), g);
-                Elem<T>::unpack(to_uint4(chunk_at(buffer_row(it), cc)), d);
+                Elem<T>::unpack(to_uint4(dv[it]), d);
 #pragma unroll
                 for (int q = 0; q < PV; ++q) {
                     const float sg = sigmoid_fast(g[q]);
