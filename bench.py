@@ -29,11 +29,11 @@ PEAK_HBM_BYTES = 8.0e12
 # HBM-side bytes per launch of the grouped GEMM kernels at this workload, from rocprofv3 FETCH_SIZE (x 2.0) and
 # WRITE_SIZE (x 1.0), the factors a plain 1 GiB copy gives; see profiles/moe_c2_bench_rocprofv3.txt
 MEASURED_TRAFFIC_BYTES = {
-    "xma_grouped_gemm/MT": (2241106 * 2.0 + 1978368) * 1024,
-    "xma_grouped_gemm/TN+swiglu": (3853520 * 2.0 + 1399240) * 1024,
-    "xma_grouped_gemm/TN": (2044096 * 2.0 + 202115) * 1024,
-    "xma_grouped_gemm/NN+swiglu_bwd": (2395224 * 2.0 + 936641) * 1024,
-    "xma_grouped_gemm/NN": (4167404 * 2.0 + 197896) * 1024,
+    "xma_grouped_gemm/MT": (2079363 * 2.0 + 1376256) * 1024,
+    "xma_grouped_gemm/TN+swiglu": (3903522 * 2.0 + 1399238) * 1024,
+    "xma_grouped_gemm/TN": (2050466 * 2.0 + 199423) * 1024,
+    "xma_grouped_gemm/NN+swiglu_bwd": (2409304 * 2.0 + 917504) * 1024,
+    "xma_grouped_gemm/NN": (4182257 * 2.0 + 196616) * 1024,
 }
 
 WORKLOAD = {

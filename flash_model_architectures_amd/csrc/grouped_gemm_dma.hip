@@ -472,6 +472,16 @@ struct Kernel {
         const int64_t num_stages = (red_len + BK - 1) / BK;
         if (num_stages > 0) {
             Pipe::prologue(*this);
+            // Weight-gradient kind: materialise the zeroed accumulators in their registers here, while the first
+            // loads are on their way.  Measured effect on the register allocation of this instantiation: no
+            // accumulator is parked in scratch memory around the last, partial trip round the ring any more
+            // (the row-grouped kinds do not park any, and get worse with the same pin).
+            if constexpr (KIND == XMA_GEMM_MT) {
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) asm volatile("" : "+a"(acc[mi][ni]));
+            }
             wait_vmcnt<Pipe::PROLOGUE_WAIT>();
             block_barrier();
             // The two loops issue the same loads and meet at the same barriers, so waves of one work-group may
@@ -656,13 +666,19 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     constexpr int C_CHUNKS = BN / PV;             // 32
     constexpr int ROW_STEP = THREADS / C_CHUNKS;  // 8
     constexpr int IT = 64 / ROW_STEP;             // 8
-    const int cc = tid % C_CHUNKS;
-    auto buffer_row = [&](int it) { return tid / C_CHUNKS + it * ROW_STEP; };
+    // Per-lane coordinates are derived from a fresh, opaque copy of the thread index: derived from `tid` they
+    // would be the values computed before the main loop, which the compiler then keeps in scratch memory
+    // across the loop and reloads in the middle of the epilogue's batched requests.
+    const int etid = opaque(tid);
+    const int cc = etid % C_CHUNKS;
+    auto buffer_row = [&](int it) { return etid / C_CHUNKS + it * ROW_STEP; };
     auto tile_row = [&](int mi, int br) { return (br >> 5) * 128 + mi * 32 + (br & 31); };
 
     int32_t orow[MI][IT];  // output row of each owned row, -1: past the end of the expert's rows
+    // Branch-free: rows past the end read the index of the expert's last row and are marked afterwards.  (Putting
+    // off the marking until the accumulators have gone to LDS, to overlap the index loads with that copy,
+    // measured no gain.)
     if constexpr (KIND != XMA_GEMM_MT) {
-        // branch-free: rows past the end read the index of the expert's last row and are then marked
         const int64_t last = m_end - 1;
         auto fill = [&](auto index_of) {
 #pragma unroll
@@ -682,34 +698,37 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                     orow[mi][it] = p < m_end ? orow[mi][it] : -1;
                 }
         };
-        if (P.out_index == nullptr) fill([&](int64_t p) { return (int32_t)p; });
-        else if (P.idx_is_i64) fill([&](int64_t p) { return (int32_t)reinterpret_cast<const int64_t*>(P.out_index)[p]; });
-        else fill([&](int64_t p) { return reinterpret_cast<const int32_t*>(P.out_index)[p]; });
+        if (EPI == XMA_EPI_SWIGLU_BWD || P.out_index == nullptr)  // that epilogue only writes grouped rows
+            fill([&](int64_t p) { return (int32_t)p; });
+        else if (P.idx_is_i64)
+            fill([&](int64_t p) { return (int32_t)reinterpret_cast<const int64_t*>(P.out_index)[p]; });
+        else
+            fill([&](int64_t p) { return reinterpret_cast<const int32_t*>(P.out_index)[p]; });
     }
 
     // SwiGLU backward: the saved pre-activation chunks (up, gate) of the rows of slab mi, double-buffered so
     // that slab mi+1 is on its way from HBM while slab mi is processed
     constexpr bool SWBWD = EPI == XMA_EPI_SWIGLU_BWD;
     u32x4_t hu[SWBWD ? 2 : 1][IT], hg[SWBWD ? 2 : 1][IT];
-    auto load_saved = [&](int mi, u32x4_t (&up)[IT], u32x4_t (&gate)[IT], const int32_t (&out_row)[IT]) {
+    auto load_saved = [&](int mi, u32x4_t (&up)[IT], u32x4_t (&gate)[IT]) {
         // branch-free: rows / columns outside the tile's part of the operand re-read a valid chunk
         const int64_t n = n0 + cc * PV < P.n ? n0 + cc * PV : 0;
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
             const int64_t p = m_begin + tile_row(mi, buffer_row(it));
-            const T* h = reinterpret_cast<const T*>(P.aux) + (out_row[it] >= 0 ? p : m_end - 1) * P.ld_aux;
+            const T* h = reinterpret_cast<const T*>(P.aux) + (p < m_end ? p : m_end - 1) * P.ld_aux;
             up[it] = *reinterpret_cast<const u32x4_t*>(h + n);
             gate[it] = *reinterpret_cast<const u32x4_t*>(h + P.n + n);
         }
     };
-    if constexpr (SWBWD) load_saved(0, hu[0], hg[0], orow[0]);
+    if constexpr (SWBWD) load_saved(0, hu[0], hg[0]);
 
     // MFMA result element r of lane l: tile column 8*(r/4) + 4*(l/32) + r%4 (+32*ni), tile row l%32 (+32*mi).
     // A 512-byte LDS row holds 32 chunks of 8 columns; chunk c of buffer row br sits at c ^ (br & 31).
     {
         const int wn0 = (k.wave % WAVES_N) * WN;
-        const int br = (k.wave / WAVES_N) * 32 + (k.lane & 31);
-        const int half = k.lane >> 5;
+        const int br = (k.wave / WAVES_N) * 32 + (etid & 31);
+        const int half = (etid >> 5) & 1;
         auto write_rows = [&](char* buf, const f32x16_t (&a)[NI]) {
 #pragma unroll
             for (int ni = 0; ni < NI; ++ni) {
@@ -773,7 +792,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             u32x4_t ups[IT / 2], gates[IT / 2];
 #pragma unroll
             for (int it2 = 0; it2 < IT / 2; ++it2) {
-                const int br = tid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
+                const int br = etid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
                 ups[it2] = chunk_at(br, pair);
                 gates[it2] = chunk_at(br, pair + HALF_CHUNKS);
             }
@@ -786,7 +805,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 #pragma unroll
             for (int it2 = 0; it2 < IT / 2; ++it2) {
                 const int32_t row_out = odd ? out_row[2 * it2 + 1] : out_row[2 * it2];
-                const int br = tid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
+                const int br = etid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
                 if (row_out < 0 || j >= half_n) continue;
                 const int64_t p = m_begin + tile_row(mi, br);
                 const u32x4_t up = ups[it2], gate = gates[it2];
@@ -804,7 +823,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             }
         } else {  // XMA_EPI_SWIGLU_BWD
             const int64_t n = n0 + cc * PV;
-            if constexpr (mi + 1 < MI) load_saved(mi + 1, hu[(mi + 1) & 1], hg[(mi + 1) & 1], orow[mi + 1 < MI ? mi + 1 : 0]);
+            if constexpr (mi + 1 < MI) load_saved(mi + 1, hu[(mi + 1) & 1], hg[(mi + 1) & 1]);
             u32x4_t dv[IT];
             read_own_chunks(dv);
 #pragma unroll
