@@ -36,7 +36,7 @@
 #define XMA_PIPE_NN Ring64x5
 #endif
 #ifndef XMA_PIPE_MT
-#define XMA_PIPE_MT Ring32x5
+#define XMA_PIPE_MT Ring64x5
 #endif
 
 namespace xma {
@@ -269,7 +269,8 @@ struct OperandLoads {
 // unit takes about sixteen cycles per DMA instruction and a wave that issues into a full queue stalls,
 // matrix instructions included.
 //
-// Ring32x5: stage j of 32 reduction elements lives in slab j % 5 (A tile | B tile).  At a step's barrier
+// Ring32x5 (an alternative kept selectable with -DXMA_PIPE_*=Ring32x5; every kind measured 1-2 % slower with
+// it than with Ring64x5): stage j of 32 reduction elements lives in slab j % 5 (A tile | B tile).  At a step's barrier
 // the next stage has landed and three more are in flight; the step's own slab then takes stage s+5:
 // its A tile during the rest of this step, its B tile during the first phase of the next step.
 struct Ring32x5 {
