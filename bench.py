@@ -55,7 +55,7 @@ def _parse() -> argparse.Namespace:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aux", action="store_true", help="skip the stand-alone timings of the HBM-bound kernels")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument(
         "--copy-probe",
         action="store_true",
@@ -76,6 +76,7 @@ def _cpu_baseline(moe, x, d_y, sample_tokens: int) -> dict:
     torch.set_num_threads(cores)
     k = moe.top_k
     params = [p.detach().cpu().requires_grad_() for p in (moe.gate.weight, moe.c_fc.weight, moe.c_proj.weight)]
+    sample_tokens = min(sample_tokens, x.size(0))
     xs = x.detach()[:sample_tokens].cpu().requires_grad_()
     dys = d_y[:sample_tokens].cpu()
 
