@@ -503,6 +503,7 @@ void fill_params(const xma_grouped_gemm_args& a, GemmParams& P) {
     P.c = a.c;
     P.aux = a.aux;
     P.offsets = a.expert_offsets;
+    P.expert_order = nullptr;
     P.in_index = a.in_index;
     P.out_index = a.out_index;
     P.lda = a.lda;
@@ -576,6 +577,9 @@ int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
         XMA_REQUIRE(a.epilogue == XMA_EPI_NONE, "xma_grouped_gemm: MT takes no epilogue");
         XMA_REQUIRE(a.lda >= a.n && a.ldb >= a.k && a.ldc >= a.k, "xma_grouped_gemm: MT row strides too small");
         XMA_REQUIRE(a.out_index == nullptr, "xma_grouped_gemm: MT takes no out_index");
+        XMA_REQUIRE(a.workspace == nullptr || a.workspace_bytes >= expert_order_bytes(a.num_experts),
+                    "xma_grouped_gemm: MT workspace too small (%lld < %lld)", (long long)a.workspace_bytes,
+                    (long long)expert_order_bytes(a.num_experts));
         if (a.n == 0 || a.k == 0) return 0;
     } else {
         XMA_REQUIRE(a.epilogue == XMA_EPI_NONE || (a.kind == XMA_GEMM_TN && a.epilogue == XMA_EPI_SWIGLU) ||

@@ -39,6 +39,9 @@ struct GemmParams {
     int32_t* split_counters;  // [kSplitSlots] arrivals per split tile, zero at launch
     float* split_partials;    // [kSplitSlots][tile] fp32 accumulators of the parts
     int32_t num_cu;
+    // MT: experts in descending order of their row counts, one record {expert, first row, end row, 0} per slot;
+    // nullptr: slot e is expert e
+    const int32_t* expert_order;
 };
 
 // At most kSplitSlots (tile, part) pairs exist at a time: the split tiles are those of one round of the device.
@@ -49,6 +52,43 @@ constexpr int64_t kSplitTileFloats = 256 * 256;
 inline int64_t tile_table_bytes(int64_t row_tiles) { return ((4 + 2 * row_tiles) * (int64_t)sizeof(int32_t) + 255) / 256 * 256; }
 inline int64_t split_region_bytes() {
     return kSplitSlots * (int64_t)sizeof(int32_t) + kSplitSlots * kSplitTileFloats * (int64_t)sizeof(float);
+}
+
+// The weight-gradient kind walks the experts in descending order of their row counts (ties: lower expert first), so
+// that the cost of consecutive bands of tiles falls monotonically and dealing them to the XCDs forwards and backwards
+// in turn (locate_tile<true>) gives every XCD about the same work however skewed the routing is.  One block;
+// rank sort for up to kMaxOrderedExperts experts, natural order beyond.
+constexpr int kMaxOrderedExperts = 1024;
+inline int64_t expert_order_bytes(int64_t E) { return 4 * E * (int64_t)sizeof(int32_t); }
+static __global__ __launch_bounds__(1024) void build_expert_order_kernel(const int32_t* __restrict__ offsets, int E,
+                                                                         int32_t* __restrict__ records) {
+    __shared__ int32_t count[kMaxOrderedExperts];
+    if (E > kMaxOrderedExperts) {
+        for (int e = threadIdx.x; e < E; e += blockDim.x) {
+            records[4 * e] = e;
+            records[4 * e + 1] = offsets[e];
+            records[4 * e + 2] = offsets[e + 1];
+            records[4 * e + 3] = 0;
+        }
+        return;
+    }
+    const int e = threadIdx.x;
+    int32_t begin = 0, end = 0;
+    if (e < E) {
+        begin = offsets[e];
+        end = offsets[e + 1];
+        count[e] = end - begin;
+    }
+    __syncthreads();
+    if (e < E) {
+        const int32_t mine = end - begin;
+        int slot = 0;
+        for (int o = 0; o < E; ++o) slot += (count[o] > mine || (count[o] == mine && o < e)) ? 1 : 0;
+        records[4 * slot] = e;
+        records[4 * slot + 1] = begin;
+        records[4 * slot + 2] = end;
+        records[4 * slot + 3] = 0;
+    }
 }
 
 // routed row p -> source row of the gathered operand (indices are < 2^31, so divide in 32 bits)
@@ -102,8 +142,9 @@ static __global__ __launch_bounds__(1024) void build_row_tiles_kernel(const int3
 // the same XCD.  Two ways to deal the tiles:
 //   SPREAD = false: XCD x takes the x-th of eight equal contiguous ranges of the tile sequence (ranges may
 //     cut a band).  Balanced to one tile when every tile costs the same (row-grouped kinds).
-//   SPREAD = true: XCD x takes whole bands x, x+8, x+16, ...; spreads a run of expensive bands (the
-//     weight-gradient tiles of an overloaded expert) over all XCDs.
+//   SPREAD = true: every group of eight consecutive bands is dealt one band per XCD, forwards and backwards in
+//     turn; spreads a run of expensive bands (the weight-gradient tiles of an overloaded expert) over all XCDs and,
+//     when band costs fall monotonically, balances them.
 // `row_tiles` is the number of row tiles actually present.  Returns false when this work-group has no tile.
 template <bool SPREAD>
 __device__ __forceinline__ bool locate_tile(int row_tiles, int col_tiles, int& row_tile, int& col_tile) {
@@ -112,7 +153,9 @@ __device__ __forceinline__ bool locate_tile(int row_tiles, int col_tiles, int& r
     const int per_band = kBandTiles * col_tiles;
     int band, in_band;
     if constexpr (SPREAD) {
-        band = (local / per_band) * kNumXcd + xcd;
+        // forwards over the XCDs for even groups of eight bands, backwards for odd ones
+        const int group = local / per_band;
+        band = group * kNumXcd + ((group & 1) ? kNumXcd - 1 - xcd : xcd);
         in_band = local % per_band;
     } else {
         const int total = row_tiles * col_tiles;

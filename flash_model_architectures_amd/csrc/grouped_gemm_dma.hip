@@ -524,10 +524,18 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     int expert;
     int64_t m_begin, m_end, tile_i0 = 0, n0;
     if constexpr (KIND == XMA_GEMM_MT) {
-        expert = row_tile / P.row_tiles_max;
+        const int slot = row_tile / P.row_tiles_max;
         tile_i0 = (int64_t)(row_tile % P.row_tiles_max) * BM;
-        m_begin = P.offsets[expert];
-        m_end = P.offsets[expert + 1];
+        if (P.expert_order != nullptr) {  // experts in descending order of their row counts
+            const int32_t* record = P.expert_order + 4 * slot;
+            expert = record[0];
+            m_begin = record[1];
+            m_end = record[2];
+        } else {
+            expert = slot;
+            m_begin = P.offsets[expert];
+            m_end = P.offsets[expert + 1];
+        }
         k.red_len = m_end - m_begin;
         n0 = (int64_t)col_tile * BN;
     } else {
@@ -877,6 +885,12 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
         P.row_tiles_max = (int32_t)ceil_div(a.n, BM);
         P.col_tiles = (int32_t)ceil_div(a.k, BN);
         grid = grid_for_tiles((int64_t)P.row_tiles_max * a.num_experts, P.col_tiles);
+        if (a.workspace != nullptr) {  // size checked by the caller
+            int32_t* records = reinterpret_cast<int32_t*>(a.workspace);
+            hipLaunchKernelGGL(build_expert_order_kernel, dim3(1), dim3(1024), 0, stream, a.expert_offsets,
+                               a.num_experts, records);
+            P.expert_order = records;
+        }
     } else {
         const int64_t rt = max_row_tiles(a.rows, a.num_experts, BM);
         int32_t* ws = reinterpret_cast<int32_t*>(a.workspace);

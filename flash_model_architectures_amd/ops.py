@@ -456,11 +456,12 @@ def _grouped_gemm(
     args.expert_offsets = expert_offsets.data_ptr()
     args.in_index, args.out_index = nat.ptr(in_index), nat.ptr(out_index)
     args.idx_is_i64, args.in_fan_out = _i64(index), in_fan_out
-    workspace = None
     if kind != nat.GEMM_MT:
         ws_bytes = nat.load().xma_grouped_gemm_workspace_bytes(E, rows)
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
-        args.workspace, args.workspace_bytes = workspace.data_ptr(), ws_bytes
+    else:
+        ws_bytes = 16 * E  # the expert order of the weight-gradient kernel
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
+    args.workspace, args.workspace_bytes = workspace.data_ptr(), ws_bytes
     tag = "xma_grouped_gemm/" + ("TN", "NN", "MT")[kind] + ("", "+swiglu", "+swiglu_bwd")[epilogue]
     nat.call("xma_grouped_gemm", ctypes.byref(args), nat.stream(), tag=tag, flops=2.0 * rows * n * k)
 

@@ -76,7 +76,9 @@ typedef struct xma_grouped_gemm_args {
     const void* out_index;
     int32_t idx_is_i64;
     int32_t in_fan_out;
-    void* workspace;         /* TN/NN: xma_grouped_gemm_workspace_bytes(num_experts, rows) bytes */
+    void* workspace;         /* TN/NN: xma_grouped_gemm_workspace_bytes(num_experts, rows) bytes.  MT: optional,
+                                16 * num_experts bytes; with it the 16-bit kernel walks the experts in descending
+                                order of their row counts, which balances the chip under skewed routing */
     int64_t workspace_bytes;
 } xma_grouped_gemm_args;
 

@@ -186,3 +186,29 @@ def test_whole_rounds_plus_split_remainder(layout):
     ref = torch.cat([a[off[e] : off[e + 1]].float() @ w[e].float().T for e in range(E)])
     assert_close(outs[0], ref, TOL[torch.bfloat16])
     assert torch.equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_weight_gradient_expert_order(dtype):
+    """The 16-bit weight-gradient kernel walks the experts in descending order of their row counts (ties: lower
+    expert first).  Sizes out of order, with ties and empty experts: every DW[e] must still land in slot e, and
+    the result must not depend on the order (checked against per-expert fp32 matmuls)."""
+
+    dev = "cuda"
+    sizes = [3, 700, 0, 700, 1, 0, 2500, 64, 64, 9, 1300, 0, 5, 64, 257, 31, 8, 0, 511, 2]
+    E, N, K = len(sizes), 264, 520
+    M = sum(sizes)
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    dy = torch.randn(M, N, generator=g).to(dtype)
+    off = torch.tensor([0] + list(torch.tensor(sizes).cumsum(0)), dtype=torch.int32)
+    dw = torch.full((E, N, K), float("nan"), dtype=dtype, device=dev)
+    ops.group_bwd_W(dy.to(dev), x.to(dev), off.to(dev), dw.permute(0, 2, 1), E)
+    ref = torch.stack([dy[off[e] : off[e + 1]].float().T @ x[off[e] : off[e + 1]].float() for e in range(E)])
+    assert_close(dw, ref, TOL[dtype], "weight gradient, experts out of size order")
+    for e in range(E):
+        if sizes[e] == 0:
+            assert bool(torch.all(dw[e] == 0)), f"empty expert {e} not zeroed"
+        else:
+            err = (dw[e].float().cpu() - ref[e]).abs().max() / ref[e].abs().max()
+            assert err < 10 * TOL[dtype], f"expert {e}: {err}"
