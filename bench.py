@@ -105,8 +105,8 @@ def _cpu_baseline(moe, x, d_y, sample_tokens: int) -> dict:
 
 def _aux_hbm_kernels(T: int, H: int, I: int, E: int, k: int) -> list:
     """Stand-alone timings (events on the current stream, outside the timed steps) of the HBM-bound kernels of
-    the path at this workload's sizes, plus the histogram / permutation / row moves at the sizes the survey
-    names for them (2^20 ids into 256 bins, 2^20 x 4096 bf16 rows; the histogram also at 2^28 ids, which does
+    the path at this workload's sizes, plus the histogram / permutation / row moves at fixed large sizes
+    (2^20 ids into 256 bins, 2^20 x 4096 bf16 rows; the histogram also at 2^28 ids, which does
     not fit the Infinity Cache)."""
 
     import torch
