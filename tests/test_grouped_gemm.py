@@ -212,3 +212,21 @@ def test_weight_gradient_expert_order(dtype):
         else:
             err = (dw[e].float().cpu() - ref[e]).abs().max() / ref[e].abs().max()
             assert err < 10 * TOL[dtype], f"expert {e}: {err}"
+
+
+def test_weight_gradient_many_experts_natural_order():
+    """Beyond 1024 experts the weight-gradient kernel keeps the natural expert order; same checks as above."""
+
+    dev = "cuda"
+    E, N, K = 1100, 16, 24
+    g = torch.Generator().manual_seed(5)
+    sizes = torch.randint(0, 5, (E,), generator=g).tolist()
+    sizes[7] = 300
+    M = sum(sizes)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    dy = torch.randn(M, N, generator=g).to(torch.bfloat16)
+    off = torch.tensor([0] + list(torch.tensor(sizes).cumsum(0)), dtype=torch.int32)
+    dw = torch.full((E, N, K), float("nan"), dtype=torch.bfloat16, device=dev)
+    ops.group_bwd_W(dy.to(dev), x.to(dev), off.to(dev), dw.permute(0, 2, 1), E)
+    ref = torch.stack([dy[off[e] : off[e + 1]].float().T @ x[off[e] : off[e + 1]].float() for e in range(E)])
+    assert_close(dw, ref, TOL[torch.bfloat16], "weight gradient, 1100 experts")
