@@ -29,11 +29,11 @@ PEAK_HBM_BYTES = 8.0e12
 # HBM-side bytes per launch of the grouped GEMM kernels at this workload, from rocprofv3 FETCH_SIZE (x 2.0) and
 # WRITE_SIZE (x 1.0), the factors a plain 1 GiB copy gives; see profiles/moe_c2_bench_rocprofv3.txt
 MEASURED_TRAFFIC_BYTES = {
-    "xma_grouped_gemm/MT": (2066582 * 2.0 + 1376256) * 1024,
-    "xma_grouped_gemm/TN+swiglu": (3888322 * 2.0 + 1399237) * 1024,
-    "xma_grouped_gemm/TN": (2048907 * 2.0 + 199432) * 1024,
-    "xma_grouped_gemm/NN+swiglu_bwd": (2416999 * 2.0 + 917504) * 1024,
-    "xma_grouped_gemm/NN": (4180507 * 2.0 + 196616) * 1024,
+    "xma_grouped_gemm/MT": (2079567 * 2.0 + 1376579) * 1024,
+    "xma_grouped_gemm/TN+swiglu": (3867151 * 2.0 + 1399233) * 1024,
+    "xma_grouped_gemm/TN": (2043859 * 2.0 + 199429) * 1024,
+    "xma_grouped_gemm/NN+swiglu_bwd": (2408652 * 2.0 + 917504) * 1024,
+    "xma_grouped_gemm/NN": (4181010 * 2.0 + 196616) * 1024,
 }
 
 WORKLOAD = {

