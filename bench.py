@@ -26,15 +26,39 @@ if ROOT not in sys.path:
 PEAK_BF16_FLOPS = 2.5e15
 PEAK_HBM_BYTES = 8.0e12
 
-# HBM-side bytes per launch of the grouped GEMM kernels at this workload, from rocprofv3 FETCH_SIZE (x 2.0) and
-# WRITE_SIZE (x 1.0), the factors a plain 1 GiB copy gives; see profiles/moe_c2_bench_rocprofv3.txt
-MEASURED_TRAFFIC_BYTES = {
-    "xma_grouped_gemm/MT": (2079567 * 2.0 + 1376579) * 1024,
-    "xma_grouped_gemm/TN+swiglu": (3867151 * 2.0 + 1399233) * 1024,
-    "xma_grouped_gemm/TN": (2043859 * 2.0 + 199429) * 1024,
-    "xma_grouped_gemm/NN+swiglu_bwd": (2408652 * 2.0 + 917504) * 1024,
-    "xma_grouped_gemm/NN": (4181010 * 2.0 + 196616) * 1024,
+# HBM-side bytes per launch of the grouped GEMM kernels at this workload are not measured by this script: they come
+# from two rocprofv3 --pmc runs of it (FETCH_SIZE, WRITE_SIZE), whose per-kernel averages and copy-kernel scale
+# factors are kept in the profile summary below.  `roofline.traffic` is read from that file at run time.
+TRAFFIC_PROFILE = os.path.join("profiles", "moe_c2_bench_rocprofv3.txt")
+TRAFFIC_ROW_TAGS = {
+    (2, 0): "xma_grouped_gemm/MT",
+    (0, 1): "xma_grouped_gemm/TN+swiglu",
+    (0, 0): "xma_grouped_gemm/TN",
+    (1, 2): "xma_grouped_gemm/NN+swiglu_bwd",
+    (1, 0): "xma_grouped_gemm/NN",
 }
+
+
+def _profiled_traffic_bytes() -> dict:
+    """tag -> HBM-side bytes per launch, from the table 'layout,epi  FETCH KiB  WRITE KiB' of the profile summary
+    and the scale factors it states ('FETCH_SIZE is scaled by F and WRITE_SIZE by W'); {} if the file is absent."""
+
+    import re
+
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE), encoding="utf-8").read()
+    except OSError:
+        return {}
+    scale = re.search(r"FETCH_SIZE is scaled by ([0-9.]+) and WRITE_SIZE by ([0-9.]+)", text)
+    if scale is None:
+        return {}
+    fetch_scale, write_scale = float(scale.group(1)), float(scale.group(2))
+    out = {}
+    for layout, epi, fetch_kib, write_kib in re.findall(r"^\s*(\d),\s*(\d)\s+(\d+)\s+(\d+)\s", text, flags=re.M):
+        tag = TRAFFIC_ROW_TAGS.get((int(layout), int(epi)))
+        if tag is not None:
+            out[tag] = (int(fetch_kib) * fetch_scale + int(write_kib) * write_scale) * 1024
+    return out
 
 WORKLOAD = {
     "workload": "Mixtral-shaped MoE layer, forward+backward",
@@ -48,6 +72,23 @@ WORKLOAD = {
 }
 
 
+# The other two GPU configurations of the workload definition.  They are timed after the headline region and
+# reported under "other_configs"; the headline line stays the Mixtral-shaped layer.
+OTHER_WORKLOADS = [
+    {
+        "workload": "fine-grained MoE layer, forward+backward",
+        "tokens": 16384, "hidden": 2048, "intermediate": 1024, "experts": 64, "top_k": 6,
+        "activation": "swiglu_packed", "routing": "linear gate, near-uniform expert load",
+    },
+    {
+        "workload": "skewed-routing MoE layer, forward+backward",
+        "tokens": 16384, "hidden": 2048, "intermediate": 768, "experts": 128, "top_k": 8,
+        "activation": "swiglu_packed",
+        "routing": "linear gate + bias[e] = -c * 1.2 * ln(e + 1); c raised from 1 in steps of 0.5 until >= 4 experts are empty",
+    },
+]  # fmt: skip
+
+
 def _parse() -> argparse.Namespace:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -55,6 +96,8 @@ def _parse() -> argparse.Namespace:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aux", action="store_true", help="skip the stand-alone timings of the HBM-bound kernels")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the fine-grained and skewed-routing layers")
+    ap.add_argument("--other-steps", type=int, default=10, help="timed passes of each of the other configurations")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument(
         "--copy-probe",
@@ -101,6 +144,112 @@ def _cpu_baseline(moe, x, d_y, sample_tokens: int) -> dict:
         f"1 timed iteration after 1 warm-up ({seconds:.2f} s); per-expert weight-gradient zero fills do not "
         "shrink with the sample, so the full-size rate is no lower than this",
     }
+
+
+def _kernel_table(summary: dict, steps: int) -> list:
+    """Per-kernel rows (average launch time, work rate, fraction of the bounding peak) from a Timeline summary."""
+
+    kernels = []
+    for tag, row in sorted(summary.items(), key=lambda kv: -kv[1]["ms"]):
+        avg_ms = row["ms"] / row["launches"]
+        entry = {
+            "kernel": tag,
+            "launches_per_step": row["launches"] / steps,
+            "avg_ms": round(avg_ms, 4),
+            "ms_per_step": round(row["ms"] / steps, 4),
+        }
+        if row["flops"] > 0:
+            entry["flops_per_launch"] = row["flops"] / row["launches"]
+            entry["tflops"] = round(row["flops"] / row["ms"] / 1e9, 2)
+            entry["frac_of_bf16_peak"] = round(row["flops"] / (row["ms"] * 1e-3) / PEAK_BF16_FLOPS, 4)
+        elif row["bytes"] > 0:
+            entry["gbps"] = round(row["bytes"] / row["ms"] / 1e6, 1)
+            entry["frac_of_hbm_peak"] = round(row["bytes"] / (row["ms"] * 1e-3) / PEAK_HBM_BYTES, 4)
+        kernels.append(entry)
+    return kernels
+
+
+def _other_config(workload: dict, steps: int, warmup: int) -> dict:
+    """Forward+backward of one of OTHER_WORKLOADS, timed like the headline region (host clock around `steps`
+    passes, events on the launch stream around every native call)."""
+
+    import math
+
+    import torch
+
+    import flash_model_architectures_amd as xma
+    from flash_model_architectures_amd import _native
+
+    dev, dt = torch.device("cuda:0"), torch.bfloat16
+    T, H, I = workload["tokens"], workload["hidden"], workload["intermediate"]
+    E, k = workload["experts"], workload["top_k"]
+    torch.manual_seed(0)
+    moe = xma.MoE(E, k, H, I, xma.swiglu_packed, True, False, 0.02).to(dt).to(dev)
+    x = torch.randn(T, H, device=dev).to(dt).requires_grad_()
+    d_y = torch.randn(T, H, device=dev).to(dt)
+
+    result = {"config": workload}
+    if "bias" in workload["routing"]:
+        with torch.no_grad():
+            raw = moe.gate(x)
+        zipf = -1.2 * torch.log(torch.arange(E, dtype=torch.float32, device=dev) + 1.0)
+        c = 1.0
+        while True:
+            _, selected = xma.topk_softmax(raw + (c * zipf).to(dt), k)
+            if E - int(torch.unique(selected).numel()) >= 4 or c >= 16.0:
+                break
+            c += 0.5
+        bias = (c * zipf).to(dt)
+        moe.gate.register_forward_hook(lambda mod, inp, out: out + bias)
+        result["zipf_bias_scale_c"] = c
+
+    def step() -> None:
+        y, _ = moe(x)
+        y.backward(d_y)
+        x.grad = None
+        moe.zero_grad(set_to_none=True)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    timeline = _native.Timeline()
+    _native.set_timeline(timeline)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    _native.set_timeline(None)
+
+    with torch.no_grad():
+        logits = moe.gate(x)
+        _, selected = xma.topk_softmax(logits, k)
+        counts = xma.route_tokens(selected, E).expert_frequency.cpu().to(torch.int64)
+    kernels = _kernel_table(timeline.summary(), steps)
+    gemm_ms = sum(kr["ms_per_step"] for kr in kernels if kr["kernel"].startswith("xma_grouped_gemm"))
+    flops = 18.0 * T * k * H * I
+    ms_per_step = seconds / steps * 1e3
+    result.update(
+        {
+            "tokens_per_s": round(T * steps / seconds, 1),
+            "ms_per_step": round(ms_per_step, 3),
+            "steps": steps,
+            "layer_tflops": round(flops / (ms_per_step * 1e-3) / 1e12, 2),
+            "grouped_gemm_ms_per_step": round(gemm_ms, 4),
+            "grouped_gemm_tflops": round(flops / (gemm_ms * 1e-3) / 1e12, 2) if gemm_ms else None,
+            "grouped_gemm_frac_of_bf16_peak": round(flops / (gemm_ms * 1e-3) / PEAK_BF16_FLOPS, 4) if gemm_ms else None,
+            "expert_rows": {
+                "routed_rows": int(counts.sum()),
+                "empty_experts": int((counts == 0).sum()),
+                "min": int(counts.min()),
+                "max": int(counts.max()),
+                "experts_under_256_rows": int((counts < 256).sum()),
+                "row_tiles_of_256": int(sum(math.ceil(c / 256) for c in counts.tolist())),
+            },
+            "kernels": kernels,
+        }
+    )
+    return result
 
 
 def _aux_hbm_kernels(T: int, H: int, I: int, E: int, k: int) -> list:
@@ -215,23 +364,7 @@ def main() -> int:
     tokens_per_s = T * args.steps / seconds
     gemm_flops = 18.0 * T * k * H * I  # forward 6*M*H*I, backward twice that
 
-    kernels = []
-    for tag, row in sorted(timeline.summary().items(), key=lambda kv: -kv[1]["ms"]):
-        avg_ms = row["ms"] / row["launches"]
-        entry = {
-            "kernel": tag,
-            "launches_per_step": row["launches"] / args.steps,
-            "avg_ms": round(avg_ms, 4),
-            "ms_per_step": round(row["ms"] / args.steps, 4),
-        }
-        if row["flops"] > 0:
-            entry["flops_per_launch"] = row["flops"] / row["launches"]
-            entry["tflops"] = round(row["flops"] / row["ms"] / 1e9, 2)
-            entry["frac_of_bf16_peak"] = round(row["flops"] / (row["ms"] * 1e-3) / PEAK_BF16_FLOPS, 4)
-        elif row["bytes"] > 0:
-            entry["gbps"] = round(row["bytes"] / row["ms"] / 1e6, 1)
-            entry["frac_of_hbm_peak"] = round(row["bytes"] / (row["ms"] * 1e-3) / PEAK_HBM_BYTES, 4)
-        kernels.append(entry)
+    kernels = _kernel_table(timeline.summary(), args.steps)
 
     dominant = kernels[0]
     if "tflops" in dominant:
@@ -242,7 +375,9 @@ def main() -> int:
             "peak": PEAK_BF16_FLOPS / 1e12,
             "unit": "TFLOP/s",
             "frac": dominant["frac_of_bf16_peak"],
-            "traffic": MEASURED_TRAFFIC_BYTES.get(dominant["kernel"]),
+            "traffic": _profiled_traffic_bytes().get(dominant["kernel"]),
+            "traffic_source": TRAFFIC_PROFILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script; "
+            "read from that file, not measured in this run)",
             "algorithmic_flops_per_launch": dominant["flops_per_launch"],
         }
     else:
@@ -277,6 +412,8 @@ def main() -> int:
         "roofline": roofline,
         "kernels": kernels,
     }
+    if not args.no_other_configs:
+        result["other_configs"] = [_other_config(w, args.other_steps, 2) for w in OTHER_WORKLOADS]
     if not args.no_aux:
         result["aux_hbm_kernels"] = _aux_hbm_kernels(T, H, I, E, k)
     if not args.no_cpu_baseline:

@@ -183,7 +183,7 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
     // ---- which tile ----
     const int row_tiles = KIND == XMA_GEMM_MT ? P.row_tiles_max * P.num_experts : P.tile_count[0];
     int row_tile, col_tile;
-    if (!locate_tile<XMA_SPREAD(KIND)>(row_tiles, P.col_tiles, row_tile, col_tile)) return;
+    if (!locate_tile<KIND == XMA_GEMM_MT>(row_tiles, P.col_tiles, row_tile, col_tile)) return;
 
     const T* A = reinterpret_cast<const T*>(P.a);
     const T* B = reinterpret_cast<const T*>(P.b);
@@ -483,15 +483,13 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
     XMA_REQUIRE(grid < ((int64_t)1 << 31), "xma_grouped_gemm: %lld tiles exceed the grid limit", (long long)grid);
     (void)PV;
     auto kernel = grouped_gemm_kernel<T, KIND, EPI>;
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<T>());
-        if (err != hipSuccess) {
-            set_error("xma_grouped_gemm: cannot reserve %d bytes of LDS: %s", lds_bytes<T>(), hipGetErrorString(err));
-            return 2;
-        }
-        attr_set = true;
+    // set on every launch: the attribute belongs to the (function, device) pair, and the call is a cheap host-side
+    // update that needs no shared flag between threads
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<T>());
+    if (err != hipSuccess) {
+        set_error("xma_grouped_gemm: cannot reserve %d bytes of LDS: %s", lds_bytes<T>(), hipGetErrorString(err));
+        return 2;
     }
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(Cfg::THREADS), lds_bytes<T>(), stream, P);
     return check_launch("xma_grouped_gemm");

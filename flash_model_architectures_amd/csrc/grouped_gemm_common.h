@@ -14,10 +14,6 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // 16 bytes moved
 constexpr int kNumXcd = 8;     // accelerator complex dies, each with a private L2
 constexpr int kBandTiles = 4;  // row tiles per band of the tile walk
 
-#ifndef XMA_SPREAD
-#define XMA_SPREAD(KIND) ((KIND) == XMA_GEMM_MT)
-#endif
-
 // ---- kernel arguments -----------------------------------------------------------------------------
 struct GemmParams {
     const void* a;

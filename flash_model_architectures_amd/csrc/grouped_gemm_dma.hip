@@ -29,16 +29,6 @@
 
 #include "grouped_gemm_common.h"
 
-#ifndef XMA_PIPE_TN
-#define XMA_PIPE_TN Ring64x5
-#endif
-#ifndef XMA_PIPE_NN
-#define XMA_PIPE_NN Ring64x5
-#endif
-#ifndef XMA_PIPE_MT
-#define XMA_PIPE_MT Ring64x5
-#endif
-
 namespace xma {
 namespace dma {
 
@@ -269,32 +259,6 @@ struct OperandLoads {
 // unit takes about sixteen cycles per DMA instruction and a wave that issues into a full queue stalls,
 // matrix instructions included.
 //
-// Ring32x5 (an alternative kept selectable with -DXMA_PIPE_*=Ring32x5; every kind measured 1-2 % slower with
-// it than with Ring64x5): stage j of 32 reduction elements lives in slab j % 5 (A tile | B tile).  At a step's barrier
-// the next stage has landed and three more are in flight; the step's own slab then takes stage s+5:
-// its A tile during the rest of this step, its B tile during the first phase of the next step.
-struct Ring32x5 {
-    static constexpr int BK = 32, CYCLE = 5, KK = 2;
-    static constexpr int L = Geometry<BK>::LOADS;
-    static constexpr int PHASE_LOADS = L;
-    static constexpr int WAIT = 6 * L;           // loads that may stay in flight at a step's barrier
-    static constexpr int PROLOGUE_WAIT = 7 * L;  // ... and when the first stage is needed
-    template <int P> struct At {
-        static constexpr int A_SLAB = P, A_OFF = 0, B_SLAB = P, B_OFF = Geometry<BK>::TILE_BYTES;
-    };
-    template <typename K> __device__ static __forceinline__ void prologue(K& k) {
-        k.template issue_a<0, 0, L>(0); k.template issue_b<0, 0, L>(0);
-        k.template issue_a<1, 0, L>(1); k.template issue_b<1, 0, L>(1);
-        k.template issue_a<2, 0, L>(2); k.template issue_b<2, 0, L>(2);
-        k.template issue_a<3, 0, L>(3); k.template issue_b<3, 0, L>(3);
-        k.template issue_a<4, 0, L>(4);
-    }
-    template <int P, int PH, typename K> __device__ static __forceinline__ void issue_phase(K& k, int64_t s) {
-        if constexpr (PH == 0) k.template issue_b<(P + 4) % CYCLE, 0, L>(s + 4);
-        else k.template issue_a<P, 0, L>(s + 5);
-    }
-};
-
 // Ring64x5: stage j of 64 reduction elements keeps its A tile in slab (2j) % 5 and its B tile in slab
 // (2j + 1) % 5, so every DMA instruction of a K-contiguous operand asks for whole 128-byte lines.  At a
 // step's barrier the next stage has landed and the A tile of the one after is in flight.  The step's own
@@ -866,16 +830,13 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 // Compute units of the current device, rounded down to a multiple of the XCD count and capped at the
 // number of split slots (the split-K scheme treats that many tiles as one round).
 static int compute_units() {
-    // queried once (thread-safe initialisation of a function-local static); one device model per process
-    static const int cached = [] {
-        int device = 0, count = 0;
-        if (hipGetDevice(&device) != hipSuccess ||
-            hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count < kNumXcd)
-            count = kSplitSlots;
-        count = count > kSplitSlots ? kSplitSlots : count;
-        return count / kNumXcd * kNumXcd;
-    }();
-    return cached;
+    // asked of the calling thread's current device on every launch (a host-side attribute lookup)
+    int device = 0, count = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count < kNumXcd)
+        count = kSplitSlots;
+    count = count > kSplitSlots ? kSplitSlots : count;
+    return count / kNumXcd * kNumXcd;
 }
 
 template <typename T, int KIND, int EPI, typename Pipe>
@@ -920,9 +881,9 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
 
 template <typename T>
 static int dispatch(const xma_grouped_gemm_args& a, hipStream_t stream) {
-    using PipeTN = XMA_PIPE_TN;
-    using PipeNN = XMA_PIPE_NN;
-    using PipeMT = XMA_PIPE_MT;
+    using PipeTN = Ring64x5;
+    using PipeNN = Ring64x5;
+    using PipeMT = Ring64x5;
     switch (a.kind) {
         case XMA_GEMM_TN:
             if (a.epilogue == XMA_EPI_SWIGLU) return launch<T, XMA_GEMM_TN, XMA_EPI_SWIGLU, PipeTN>(a, stream);

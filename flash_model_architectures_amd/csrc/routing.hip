@@ -184,6 +184,24 @@ __global__ __launch_bounds__(1024) void offsets_kernel(const uint32_t* __restric
     if (threadIdx.x == 1023) offsets[E] = (int32_t)part[1023];
 }
 
+// offsets[e] = first grouped position whose expert id is >= e, for e in [0, E]: the exclusive prefix sums of the
+// histogram, recovered from the sorted ids alone.  Thread p looks at the boundary between positions p - 1 and p
+// (position -1 counts as expert -1, position n as expert E) and writes the offsets of the experts that start there,
+// so every offsets[e] is written exactly once when the ids are sorted.
+template <typename IdT>
+__global__ __launch_bounds__(256) void offsets_from_sorted_kernel(const IdT* __restrict__ sorted_ids, int64_t n, int E,
+                                                                   int32_t* __restrict__ offsets) {
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p > n) return;
+    auto clamped = [&](int64_t i) {
+        const int64_t e = (int64_t)sorted_ids[i];
+        return e < 0 ? (int64_t)0 : e > E - 1 ? (int64_t)(E - 1) : e;
+    };
+    const int64_t prev = p == 0 ? -1 : clamped(p - 1);
+    const int64_t cur = p == n ? E : clamped(p);
+    for (int64_t e = prev + 1; e <= cur; ++e) offsets[e] = (int32_t)p;
+}
+
 template <typename IdT, typename OutT>
 __global__ __launch_bounds__(256) void place_kernel(const IdT* __restrict__ ids, int64_t n, int E, int nbits,
                                                      int waves_per_block, const uint32_t* __restrict__ unit_prefix,
@@ -423,16 +441,11 @@ int64_t xma_route_workspace_bytes(int64_t n, int32_t num_experts) {
     return units * (int64_t)num_experts * (int64_t)sizeof(uint32_t);
 }
 
-int xma_route_build(const void* ids, int ids_is_i64, int64_t n, int32_t E, uint32_t* counts, int32_t* offsets,
-                    void* sorted_ids, void* perm, int out_is_i64, void* workspace, int64_t workspace_bytes,
-                    void* stream_) {
-    hipStream_t stream = (hipStream_t)stream_;
-    XMA_REQUIRE(E >= 1 && E <= kMaxExperts, "xma_route_build: num_experts=%d outside [1, %d]", E, kMaxExperts);
-    XMA_REQUIRE(n >= 0 && n < ((int64_t)1 << 31), "xma_route_build: n=%lld does not fit int32", (long long)n);
-    XMA_REQUIRE(counts && offsets, "xma_route_build: counts/offsets must not be null");
-    XMA_REQUIRE(n == 0 || (ids && sorted_ids && perm && workspace), "xma_route_build: null pointer");
-    XMA_REQUIRE(workspace_bytes >= xma_route_workspace_bytes(n, E), "xma_route_build: workspace too small (%lld < %lld)",
-                (long long)workspace_bytes, (long long)xma_route_workspace_bytes(n, E));
+// Launches of the counting sort; arguments already validated.  Every word of `workspace` that is read has been
+// written by an earlier kernel of the same call, so the workspace needs no clearing.
+static int route_build_launch(const void* ids, int ids_is_i64, int64_t n, int32_t E, uint32_t* counts,
+                              int32_t* offsets, void* sorted_ids, void* perm, int out_is_i64, void* workspace,
+                              hipStream_t stream) {
     if (n == 0) {
         hipLaunchKernelGGL(fill_u32_kernel, dim3((E + 255) / 256), dim3(256), 0, stream, counts, (int64_t)E, 0u);
         hipLaunchKernelGGL(fill_u32_kernel, dim3((E + 1 + 255) / 256), dim3(256), 0, stream, (uint32_t*)offsets,
@@ -471,6 +484,35 @@ int xma_route_build(const void* ids, int ids_is_i64, int64_t n, int32_t E, uint3
     }
 #undef XMA_PLACE
     return check_launch("xma_route_build");
+}
+
+int xma_route_build(const void* ids, int ids_is_i64, int64_t n, int32_t E, uint32_t* counts, int32_t* offsets,
+                    void* sorted_ids, void* perm, int out_is_i64, void* workspace, int64_t workspace_bytes,
+                    void* stream_) {
+    XMA_REQUIRE(E >= 1 && E <= kMaxExperts, "xma_route_build: num_experts=%d outside [1, %d]", E, kMaxExperts);
+    XMA_REQUIRE(n >= 0 && n < ((int64_t)1 << 31), "xma_route_build: n=%lld does not fit int32", (long long)n);
+    XMA_REQUIRE(counts && offsets, "xma_route_build: counts/offsets must not be null");
+    XMA_REQUIRE(n == 0 || (ids && sorted_ids && perm && workspace), "xma_route_build: null pointer");
+    XMA_REQUIRE(workspace_bytes >= xma_route_workspace_bytes(n, E), "xma_route_build: workspace too small (%lld < %lld)",
+                (long long)workspace_bytes, (long long)xma_route_workspace_bytes(n, E));
+    return route_build_launch(ids, ids_is_i64, n, E, counts, offsets, sorted_ids, perm, out_is_i64, workspace,
+                              (hipStream_t)stream_);
+}
+
+int xma_offsets_from_sorted(const void* sorted_ids, int ids_is_i64, int64_t n, int32_t E, int32_t* offsets,
+                            void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    XMA_REQUIRE(E >= 1 && E <= kMaxExperts, "xma_offsets_from_sorted: num_experts=%d outside [1, %d]", E, kMaxExperts);
+    XMA_REQUIRE(n >= 0 && n < ((int64_t)1 << 31), "xma_offsets_from_sorted: n=%lld does not fit int32", (long long)n);
+    XMA_REQUIRE(offsets != nullptr && (sorted_ids != nullptr || n == 0), "xma_offsets_from_sorted: null pointer");
+    const unsigned blocks = (unsigned)ceil_div(n + 1, 256);
+    if (ids_is_i64)
+        hipLaunchKernelGGL(offsets_from_sorted_kernel<int64_t>, dim3(blocks), dim3(256), 0, stream,
+                           (const int64_t*)sorted_ids, n, (int)E, offsets);
+    else
+        hipLaunchKernelGGL(offsets_from_sorted_kernel<int32_t>, dim3(blocks), dim3(256), 0, stream,
+                           (const int32_t*)sorted_ids, n, (int)E, offsets);
+    return check_launch("xma_offsets_from_sorted");
 }
 
 int xma_topk_softmax(const void* logits, int dtype, int64_t T, int32_t E, int32_t k, int64_t ld, void* weights,

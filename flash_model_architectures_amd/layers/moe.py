@@ -23,6 +23,7 @@ from ..functional.routing import route_tokens, topk_softmax
 from ..functional.swiglu_packed import swiglu_packed
 from ..ops import (
     add_expert_bias,
+    exclusive_offsets,
     combine_topk,
     down_projection_dgrad_swiglu,
     expert_colsum,
@@ -93,7 +94,7 @@ class _ScatteredExperts(torch.autograd.Function):
         k, grouped_in, grouped_out = ctx.k, ctx.grouped_in, ctx.grouped_out
         E, K, N = W.shape
         M = sorted_expert_idxs.size(0)
-        if grad_out.stride(-1) != 1:
+        if not grad_out.is_contiguous():  # e.g. the expanded (stride 0) gradient of y.sum() or y.mean(0)
             grad_out = grad_out.contiguous()
 
         d_gates = None
@@ -167,8 +168,11 @@ def scattered_experts(
     bias: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Same call as the reference's `scattered_experts` (triton_implementation/__init__.py:164-185) plus an
-    optional per-expert bias [E, out_features], which the reference offers on its torch path only."""
+    optional per-expert bias [E, out_features], which the reference offers on its torch path only.
+    `expert_offsets` may be the reference's inclusive cumsum of length E (xma/layers/moe/__init__.py:225) or the
+    int32[E + 1] exclusive prefix sums the kernels read; the former is converted on the device."""
 
+    expert_offsets = exclusive_offsets(expert_offsets, expert_weights.size(0))
     return _ScatteredExperts.apply(
         inputs,
         expert_weights,
@@ -229,7 +233,7 @@ class _SwigluExperts(torch.autograd.Function):
         E, I2, _ = w_up.shape
         k = gates.size(1)
         M = T * k
-        if grad_out.stride(-1) != 1:
+        if not grad_out.is_contiguous():  # e.g. the expanded (stride 0) gradient of y.sum() or y.mean(0)
             grad_out = grad_out.contiguous()
 
         d_gates = torch.empty_like(gates, memory_format=torch.contiguous_format)
@@ -319,6 +323,65 @@ class Experts(XMAModule):
             grouped_out=grouped_out,
             bias=self.bias,
         )
+
+    def up_projection_triton_forward(
+        self,
+        input: torch.Tensor,
+        num_experts_per_token: int | None = None,
+        sorted_expert_idxs: torch.Tensor | None = None,
+        sorted_scattered_idxs: torch.Tensor | None = None,
+        expert_offsets: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        """The reference's name for the up-projection call (xma/layers/moe/__init__.py:46-68): tokens in
+        scattered order in, routed rows in grouped order out.  Runs the HIP kernels; a bias is applied."""
+
+        return self.grouped_forward(
+            input, num_experts_per_token, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets,
+            gates=None, grouped_in=False, grouped_out=True,
+        )  # fmt: skip
+
+    def down_projection_triton_forward(
+        self,
+        input: torch.Tensor,
+        num_experts_per_token: int | None = None,
+        sorted_expert_idxs: torch.Tensor | None = None,
+        sorted_scattered_idxs: torch.Tensor | None = None,
+        expert_offsets: torch.Tensor | None = None,
+        gates: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        """The reference's name for the down-projection call (xma/layers/moe/__init__.py:70-93): grouped rows
+        in, tokens out, the top-k results of a token combined with `gates`."""
+
+        return self.grouped_forward(
+            input, num_experts_per_token, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets,
+            gates=gates, grouped_in=True, grouped_out=False,
+        )  # fmt: skip
+
+    def torch_forward(
+        self, input: torch.Tensor | list[torch.Tensor], expert_frequency: torch.Tensor | None, return_list: bool = False
+    ) -> list[torch.Tensor] | torch.Tensor:
+        """Call-compatible with the reference's per-expert `F.linear` loop (xma/layers/moe/__init__.py:95-111):
+        rows grouped by expert in (one tensor plus the histogram, or a list with one tensor per expert), the
+        projected rows out.  Here it is one grouped GEMM on the device; like the reference's, it reads the
+        histogram on the host when it has to split the result into a list."""
+
+        if isinstance(input, torch.Tensor):
+            sizes = expert_frequency.to(torch.int64)
+        else:
+            assert expert_frequency is None
+            sizes = torch.tensor([t.size(0) for t in input], dtype=torch.int64, device=input[0].device)
+            input = torch.cat(list(input), dim=0)
+        assert sizes.numel() == self.num_experts
+        rows = input.size(0)
+        expert_offsets = sizes.cumsum(0)
+        positions = torch.arange(rows, device=input.device, dtype=torch.int64)
+        sorted_expert_idxs = torch.searchsorted(expert_offsets, positions, right=True)
+        output = self.grouped_forward(
+            input, 1, sorted_expert_idxs, positions, expert_offsets, gates=None, grouped_in=True, grouped_out=True
+        )
+        if return_list:
+            return list(output.split(sizes.tolist(), dim=0))
+        return output
 
     def extra_repr(self) -> str:
         return f"num_experts={self.num_experts}, in_features={self.in_features}, out_features={self.out_features}"

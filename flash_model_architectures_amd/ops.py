@@ -6,9 +6,10 @@ allocates outputs with torch, the operator mutates them and returns None, so the
 owns memory.  Names and argument meaning follow the reference operators they replace; where the
 reference has a `_cuda` suffix the operator here ends in `_rocm`.
 
-`expert_offsets` is always the int32 vector of E+1 exclusive prefix sums (leading 0).  The
-reference passes the inclusive cumsum of length E (xma/layers/moe/__init__.py:225); the exclusive
-form is the same data with the implicit 0 stored.
+The kernels take `expert_offsets` as the int32 vector of E+1 exclusive prefix sums (leading 0).  The
+reference passes the inclusive cumsum of length E (xma/layers/moe/__init__.py:225), which is the same
+data without the leading 0; operators that receive that form convert it on the device, and
+`scatter2scatter`, which the reference calls without offsets, derives them from the sorted expert ids.
 """
 
 from __future__ import annotations
@@ -42,6 +43,46 @@ def _row_stride(t: torch.Tensor) -> int:
 def _check_offsets(expert_offsets: torch.Tensor, E: int) -> None:
     assert expert_offsets.dtype == torch.int32 and expert_offsets.is_contiguous()
     assert expert_offsets.numel() == E + 1, "expert_offsets must hold E + 1 exclusive prefix sums"
+
+
+def exclusive_offsets(expert_offsets: torch.Tensor, E: int) -> torch.Tensor:
+    """int32[E + 1] exclusive prefix sums from either form of the offsets: the E + 1 exclusive sums pass
+    through; the reference's length-E inclusive cumsum (any integer dtype, xma/layers/moe/__init__.py:225)
+    gets its leading 0 on the device."""
+
+    assert expert_offsets.dim() == 1, "expert_offsets must be a vector"
+    if expert_offsets.numel() == E + 1:
+        if expert_offsets.dtype != torch.int32 or not expert_offsets.is_contiguous():
+            expert_offsets = expert_offsets.to(torch.int32).contiguous()
+        return expert_offsets
+    assert expert_offsets.numel() == E, "expert_offsets must hold E inclusive or E + 1 exclusive prefix sums"
+    out = torch.zeros(E + 1, dtype=torch.int32, device=expert_offsets.device)
+    out[1:] = expert_offsets
+    return out
+
+
+# One workspace per (device, stream), grown on demand and reused by every launch on that stream: launches on a
+# stream run in order, and every kernel initialises the part of the workspace it reads.
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), nat.stream())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def offsets_from_sorted(sorted_expert_idxs: torch.Tensor, E: int) -> torch.Tensor:
+    """int32[E + 1] exclusive prefix sums of the expert histogram, from the sorted expert ids alone."""
+
+    nat.require_device(sorted_expert_idxs)
+    ids = sorted_expert_idxs.contiguous()
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=ids.device)
+    nat.call("xma_offsets_from_sorted", ids.data_ptr(), _i64(ids), ids.numel(), E, offsets.data_ptr(), nat.stream())
+    return offsets
 
 
 # ------------------------------------------------------------------------------------------------
@@ -86,7 +127,7 @@ def route_build_rocm(
     assert sorted_expert_idxs.numel() == n and sorted_scattered_idxs.numel() == n
     assert sorted_expert_idxs.is_contiguous() and sorted_scattered_idxs.is_contiguous()
     ws_bytes = nat.load().xma_route_workspace_bytes(n, E)
-    workspace = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=ids.device)
+    workspace = _workspace(ids.device, max(ws_bytes, 4))
     nat.call(
         "xma_route_build",
         ids.data_ptr(),
@@ -460,8 +501,8 @@ def _grouped_gemm(
         ws_bytes = nat.load().xma_grouped_gemm_workspace_bytes(E, rows)
     else:
         ws_bytes = 16 * E  # the expert order of the weight-gradient kernel
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
-    args.workspace, args.workspace_bytes = workspace.data_ptr(), ws_bytes
+    workspace = _workspace(a.device, ws_bytes)
+    args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
     tag = "xma_grouped_gemm/" + ("TN", "NN", "MT")[kind] + ("", "+swiglu", "+swiglu_bwd")[epilogue]
     nat.call("xma_grouped_gemm", ctypes.byref(args), nat.stream(), tag=tag, flops=2.0 * rows * n * k)
 
@@ -483,17 +524,20 @@ def scatter2scatter(
     W: torch.Tensor,
     sorted_expert_idxs: torch.Tensor,
     sorted_scattered_idxs: torch.Tensor,
-    expert_offsets: torch.Tensor,
     out: torch.Tensor,
     FAN_OUT: int,
     x_grouped: bool = False,
     y_grouped: bool = False,
+    expert_offsets: torch.Tensor | None = None,
 ) -> None:
     """out[o(p)] = X[i(p)] @ W[e(p)] over the grouped positions p.
 
     i(p) = p if x_grouped else idx[p] // FAN_OUT; o(p) = p if y_grouped else idx[p]
     (xma/layers/moe/triton_implementation/scatter_kernel.py:105-108,128-131).  W is the logical
-    [E, K, N] tensor; a permuted view of [E, N, K] storage is read in place.
+    [E, K, N] tensor; a permuted view of [E, N, K] storage is read in place.  The first eight parameters
+    are the reference operator's (scatter_kernel.py:137-147); `expert_offsets` is an optional extra (either
+    form, see `exclusive_offsets`) that saves the small kernel which otherwise recovers the offsets from
+    `sorted_expert_idxs`.
     """
 
     assert sorted_scattered_idxs.size(0) == sorted_expert_idxs.size(0)
@@ -503,6 +547,10 @@ def scatter2scatter(
     assert X.size(1) == W.size(1) and X.dtype == W.dtype == out.dtype
     kind, ldb = _weight_layout(W)
     idx = sorted_scattered_idxs.contiguous()
+    if expert_offsets is None:
+        expert_offsets = offsets_from_sorted(sorted_expert_idxs, W.size(0))
+    else:
+        expert_offsets = exclusive_offsets(expert_offsets, W.size(0))
     _grouped_gemm(
         kind=kind,
         epilogue=nat.EPI_NONE,
@@ -544,6 +592,7 @@ def group_bwd_W(
 
     assert DW.dim() == 3 and DW.size(0) == E and DW.size(1) == X.size(1) and DW.size(2) == DY.size(1)
     assert DY.dtype == X.dtype == DW.dtype
+    expert_offsets = exclusive_offsets(expert_offsets, E)
     rows = DY.size(0)
     if x_index is not None:
         x_index = x_index.contiguous()

@@ -114,6 +114,15 @@ int xma_route_build(const void* ids, int ids_is_i64, int64_t n, int32_t num_expe
                     int out_is_i64, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * offsets[e] = first position of sorted_ids (int32 or int64, non-decreasing, values in [0, num_experts)) whose
+ * value is >= e, for e in [0, num_experts]: the int32[num_experts + 1] exclusive prefix sums that xma_grouped_gemm
+ * takes, recovered from the sorted expert ids.  For callers that hold what the reference's scatter2scatter is given
+ * (xma/layers/moe/triton_implementation/scatter_kernel.py:137-147: the sorted ids, no offsets).
+ */
+int xma_offsets_from_sorted(const void* sorted_ids, int ids_is_i64, int64_t n, int32_t num_experts,
+                            int32_t* offsets, void* stream);
+
+/*
  * Router selection: for each of T rows of logits[T, E] (row stride ld) pick the k largest
  * (ties: lower expert index first; output ordered by descending value, then ascending index;
  * NaN ranks above +inf), and softmax over the k selected values in fp32

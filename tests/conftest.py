@@ -27,3 +27,23 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Worst parity figures of the session per tolerance class: whole tensor, and element-wise."""
+
+    from tests import helpers
+
+    by_tol: dict = {}
+    for what, tol, err, elem, floor in helpers.WORST:
+        cur = by_tol.setdefault((tol, floor), [0.0, "", 0.0, ""])
+        if err > cur[0]:
+            cur[0], cur[1] = err, what
+        if elem > cur[2]:
+            cur[2], cur[3] = elem, what
+    for tol, floor in sorted(by_tol):
+        err, what_err, elem, what_elem = by_tol[(tol, floor)]
+        terminalreporter.write_line(
+            f"parity, bar {tol:.0e}: worst whole-tensor error {err:.2e} ({what_err}), worst element-wise error "
+            f"|a-b| / (|b| + {floor:g} rms) {elem:.2e} ({what_elem}) against {2 * tol:.0e}"
+        )

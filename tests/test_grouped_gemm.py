@@ -56,7 +56,7 @@ def test_all_layouts_and_epilogues(case, dtype):
 
     # TN with row gather: h = x[idx // k] @ W1[e]^T, grouped output
     h = torch.empty(M, 2 * I, dtype=dtype, device=dev)
-    ops.scatter2scatter(xd, w1d.permute(0, 2, 1), sed, idxd, offd, h, k, False, True)
+    ops.scatter2scatter(xd, w1d.permute(0, 2, 1), sed, idxd, h, k, False, True, offd)
     h_ref = _per_expert(off, lambda e, s: xg[s] @ w1[e].float().T)
     assert_close(h, h_ref, tol, "up projection")
 
@@ -72,7 +72,7 @@ def test_all_layouts_and_epilogues(case, dtype):
 
     # TN with row scatter: y_exp[idx[p]] = act[p] @ W2[e]^T
     y_exp = torch.full((M, H), float("nan"), dtype=dtype, device=dev)
-    ops.scatter2scatter(act, w2d.permute(0, 2, 1), sed, idxd, offd, y_exp, 1, True, False)
+    ops.scatter2scatter(act, w2d.permute(0, 2, 1), sed, idxd, y_exp, 1, True, False, offd)
     a32 = act.float().cpu()
     y_ref = torch.empty(M, H)
     y_ref[idx] = _per_expert(off, lambda e, s: a32[s] @ w2[e].float().T)
@@ -82,7 +82,7 @@ def test_all_layouts_and_epilogues(case, dtype):
     dyg = torch.randn(M, H, generator=g).to(dtype)
     dygd = dyg.to(dev)
     d_act = torch.empty(M, I, dtype=dtype, device=dev)
-    ops.scatter2scatter(dygd, w2d, sed, idxd, offd, d_act, 1, True, True)
+    ops.scatter2scatter(dygd, w2d, sed, idxd, d_act, 1, True, True, offd)
     d_act_ref = _per_expert(off, lambda e, s: dyg[s].float() @ w2[e].float())
     assert_close(d_act, d_act_ref, tol, "input gradient")
 
@@ -95,7 +95,7 @@ def test_all_layouts_and_epilogues(case, dtype):
 
     # NN with row scatter: dXe[idx[p]] = d_pre[p] @ W1[e]
     d_xe = torch.empty(M, H, dtype=dtype, device=dev)
-    ops.scatter2scatter(d_pre, w1d, sed, idxd, offd, d_xe, 1, True, False)
+    ops.scatter2scatter(d_pre, w1d, sed, idxd, d_xe, 1, True, False, offd)
     dp = d_pre.float().cpu()
     d_xe_ref = torch.empty(M, H)
     d_xe_ref[idx] = _per_expert(off, lambda e, s: dp[s] @ w1[e].float())
@@ -128,17 +128,17 @@ def test_argument_validation():
     se = torch.zeros(8, device=dev, dtype=torch.int32)
     off = torch.tensor([0, 8, 8], device=dev, dtype=torch.int32)
     out = torch.empty(8, 32, device=dev, dtype=torch.bfloat16)
-    ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, off, out, 1, False, True)  # sanity: valid call
+    ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, out, 1, False, True, off)  # sanity: valid call
     with pytest.raises(RuntimeError, match="multiples"):
         bad_w = torch.randn(2, 12, 64, device=dev, dtype=torch.bfloat16)
-        ops.scatter2scatter(x, bad_w.permute(0, 2, 1), se, idx, off, out[:, :12], 1, False, True)
+        ops.scatter2scatter(x, bad_w.permute(0, 2, 1), se, idx, out[:, :12], 1, False, True, off)
     with pytest.raises(RuntimeError, match="aligned"):
         shifted = torch.randn(8 * 64 + 8, device=dev, dtype=torch.bfloat16)[1 : 1 + 8 * 64].view(8, 64)
-        ops.scatter2scatter(shifted, w.permute(0, 2, 1), se, idx, off, out, 1, False, True)
+        ops.scatter2scatter(shifted, w.permute(0, 2, 1), se, idx, out, 1, False, True, off)
     with pytest.raises(AssertionError):
-        ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, off[:2], out, 1, False, True)
+        ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, out, 1, False, True, off[:1])  # neither E nor E + 1 long
     with pytest.raises(ValueError):
-        ops.scatter2scatter(x[:, :32], w.permute(0, 2, 1)[:, ::2, ::2], se, idx, off, out[:, :16], 1, False, True)
+        ops.scatter2scatter(x[:, :32], w.permute(0, 2, 1)[:, ::2, ::2], se, idx, out[:, :16], 1, False, True, off)
 
 
 def test_ragged_tail_rows_are_not_touched():
@@ -153,7 +153,7 @@ def test_ragged_tail_rows_are_not_touched():
     idx = torch.arange(T, dtype=torch.int32, device=dev)
     se = torch.cat([torch.zeros(1), torch.full((299,), 2)]).int().to(dev)
     out = torch.empty(T, N, dtype=torch.bfloat16, device=dev)
-    ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, off, out, 1, True, True)
+    ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, out, 1, True, True, off)
     ref = torch.cat([x[:1].float() @ w[0].float().T, x[1:].float() @ w[2].float().T])
     assert_close(out, ref, TOL[torch.bfloat16])
 
@@ -181,7 +181,7 @@ def test_whole_rounds_plus_split_remainder(layout):
     outs = []
     for _ in range(2):
         out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
-        ops.scatter2scatter(a, weights, se, idx, off, out, 1, True, True)
+        ops.scatter2scatter(a, weights, se, idx, out, 1, True, True, off)
         outs.append(out)
     ref = torch.cat([a[off[e] : off[e + 1]].float() @ w[e].float().T for e in range(E)])
     assert_close(outs[0], ref, TOL[torch.bfloat16])

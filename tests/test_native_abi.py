@@ -26,6 +26,7 @@ def test_header_declares_the_expected_entry_points():
     for required in [
         "xma_continuous_count",
         "xma_route_build",
+        "xma_offsets_from_sorted",
         "xma_topk_softmax",
         "xma_topk_softmax_bwd",
         "xma_gather_rows",
@@ -93,6 +94,35 @@ def test_public_surface_mirrors_the_reference_names():
                "swiglu_backward_rocm", "route_build_rocm", "topk_softmax_rocm", "pack_unpack_sequence_rocm",
                "add_expert_bias", "expert_colsum"]:
         assert hasattr(torch.ops.xma, op), f"xma::{op} is not registered"
+
+
+def test_reference_side_call_signatures():
+    """What a caller written against the reference can use unchanged: the operator's argument list
+    (xma/layers/moe/triton_implementation/scatter_kernel.py:137-147) and the `Experts` method names
+    (xma/layers/moe/__init__.py:46-111)."""
+
+    import inspect
+
+    from flash_model_architectures_amd import ops
+    from flash_model_architectures_amd.layers.moe import Experts
+
+    names = list(inspect.signature(ops.scatter2scatter).parameters)
+    assert names[:8] == ["X", "W", "sorted_expert_idxs", "sorted_scattered_idxs", "out", "FAN_OUT", "x_grouped", "y_grouped"]
+    assert inspect.signature(ops.scatter2scatter).parameters["expert_offsets"].default is None
+    assert list(inspect.signature(ops.group_bwd_W).parameters)[:5] == ["DY", "X", "expert_offsets", "DW", "E"]
+    assert list(inspect.signature(ops.group).parameters) == ["A", "sorted_expert_idxs", "out", "coeff", "fan_out"]
+    up = inspect.signature(Experts.up_projection_triton_forward).parameters
+    assert list(up) == ["self", "input", "num_experts_per_token", "sorted_expert_idxs", "sorted_scattered_idxs", "expert_offsets"]
+    down = inspect.signature(Experts.down_projection_triton_forward).parameters
+    assert list(down) == list(up) + ["gates"]
+    assert list(inspect.signature(Experts.torch_forward).parameters) == ["self", "input", "expert_frequency", "return_list"]
+    # both forms of the offsets are accepted; anything else is an error
+    inclusive = torch.tensor([2, 2, 5], dtype=torch.int64)
+    assert ops.exclusive_offsets(inclusive, 3).tolist() == [0, 2, 2, 5]
+    exclusive = torch.tensor([0, 2, 2, 5], dtype=torch.int32)
+    assert ops.exclusive_offsets(exclusive, 3) is exclusive
+    with pytest.raises(AssertionError):
+        ops.exclusive_offsets(torch.zeros(5, dtype=torch.int32), 3)
 
 
 def test_moe_module_layout_and_state_dict():
