@@ -66,6 +66,11 @@ PROTOTYPES: dict[str, tuple] = {
         [c_void_p, c_int, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_void_p],
     ),
     "xma_offsets_from_sorted": (c_int, [c_void_p, c_int, c_int64, c_int32, c_void_p, c_void_p]),
+    "xma_route_build_static_max_bytes": (c_int64, []),
+    "xma_route_build_static": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
+    ),
     "xma_topk_softmax": (
         c_int,
         [c_void_p, c_int, c_int64, c_int32, c_int32, c_int64, c_void_p, c_void_p, c_int, c_void_p],

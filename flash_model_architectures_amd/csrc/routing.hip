@@ -9,12 +9,22 @@
 // exclusive scan over the units plus an exclusive scan over the experts turn the rows into
 // the first output slot of every (unit, expert) pair; (3) every wave walks its chunk again in
 // order, ranks equal ids inside each 64-wide batch with ballots, and writes the permutation.
+#include <mutex>
+
 #include "common.h"
 
 namespace xma {
 
 constexpr int kChunk = 1024;        // ids per wave-unit of the counting sort
 constexpr int kMaxExperts = 16384;  // same limit as the reference kernel (forward.cu:12)
+
+// Working memory of xma_route_build_static, the entry point that allocates nothing: the per-chunk histograms
+// that xma_route_build keeps in its caller's workspace live here instead.  One copy per GPU, held until the
+// process ends; every call on a GPU shares it, so calls that overlap on one GPU race.  Host code never uses the
+// array's name as an address: it asks the runtime for the array's device address once per device
+// (static_scratch_for_current_device) and passes that pointer to the kernels.
+constexpr int64_t kStaticScratchWords = 262144;  // 1 MiB
+static __device__ __align__(256) uint32_t scratch[kStaticScratchWords];
 
 // ------------------------------------------------------------------------------------------
 // continuous_count
@@ -403,6 +413,32 @@ static int sort_waves_per_block(int E) {
     return w;
 }
 
+// Device address of `scratch` on the GPU that is current for the calling thread; looked up once per device
+// (each GPU holds its own copy of the array at its own address).  nullptr + error text on failure.
+static uint32_t* static_scratch_for_current_device() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex lock;
+    static uint32_t* address[kMaxDevices] = {};
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess || device < 0 || device >= kMaxDevices) {
+        set_error("xma_route_build_static: no usable current device (%s, device %d)", hipGetErrorString(err), device);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> guard(lock);
+    if (address[device] == nullptr) {
+        void* p = nullptr;
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || p == nullptr) {
+            set_error("xma_route_build_static: hipGetSymbolAddress failed on device %d: %s", device,
+                      hipGetErrorString(err));
+            return nullptr;
+        }
+        address[device] = static_cast<uint32_t*>(p);
+    }
+    return address[device];
+}
+
 }  // namespace xma
 
 using namespace xma;
@@ -513,6 +549,25 @@ int xma_offsets_from_sorted(const void* sorted_ids, int ids_is_i64, int64_t n, i
         hipLaunchKernelGGL(offsets_from_sorted_kernel<int32_t>, dim3(blocks), dim3(256), 0, stream,
                            (const int32_t*)sorted_ids, n, (int)E, offsets);
     return check_launch("xma_offsets_from_sorted");
+}
+
+int64_t xma_route_build_static_max_bytes(void) { return kStaticScratchWords * (int64_t)sizeof(uint32_t); }
+
+int xma_route_build_static(const void* ids, int ids_is_i64, int64_t n, int32_t E, uint32_t* counts, int32_t* offsets,
+                           void* sorted_ids, void* perm, int out_is_i64, void* stream_) {
+    XMA_REQUIRE(E >= 1 && E <= kMaxExperts, "xma_route_build_static: num_experts=%d outside [1, %d]", E, kMaxExperts);
+    XMA_REQUIRE(n >= 0 && n < ((int64_t)1 << 31), "xma_route_build_static: n=%lld does not fit int32", (long long)n);
+    XMA_REQUIRE(counts && offsets, "xma_route_build_static: counts/offsets must not be null");
+    XMA_REQUIRE(n == 0 || (ids && sorted_ids && perm), "xma_route_build_static: null pointer");
+    const int64_t need = xma_route_workspace_bytes(n, E);
+    XMA_REQUIRE(need <= xma_route_build_static_max_bytes(),
+                "xma_route_build_static: ceil(n / %d) * num_experts * 4 = %lld bytes of working memory exceed the built-in "
+                "%lld; use xma_route_build with a caller-owned workspace",
+                kChunk, (long long)need, (long long)xma_route_build_static_max_bytes());
+    uint32_t* workspace = static_scratch_for_current_device();
+    if (workspace == nullptr) return 2;  // error text already set
+    return route_build_launch(ids, ids_is_i64, n, E, counts, offsets, sorted_ids, perm, out_is_i64, workspace,
+                              (hipStream_t)stream_);
 }
 
 int xma_topk_softmax(const void* logits, int dtype, int64_t T, int32_t E, int32_t k, int64_t ld, void* weights,

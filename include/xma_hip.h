@@ -123,6 +123,20 @@ int xma_offsets_from_sorted(const void* sorted_ids, int ids_is_i64, int64_t n, i
                             int32_t* offsets, void* stream);
 
 /*
+ * xma_route_build without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same inputs, outputs and results as xma_route_build; the per-chunk histograms live in a 1 MiB array inside the
+ * library (xma_route_build_static_max_bytes(), one copy per GPU, held until the process ends), so the call is
+ * rejected when xma_route_workspace_bytes(n, num_experts) exceeds that.  It calls no hipMalloc / hipFree.  All
+ * calls on one GPU share the array: calls that may overlap on one GPU (two streams, two threads) race, and must
+ * use xma_route_build with a workspace each instead.
+ */
+int64_t xma_route_build_static_max_bytes(void);
+int xma_route_build_static(const void* ids, int ids_is_i64, int64_t n, int32_t num_experts,
+                           uint32_t* counts, int32_t* offsets, void* sorted_ids, void* perm,
+                           int out_is_i64, void* stream);
+
+/*
  * Router selection: for each of T rows of logits[T, E] (row stride ld) pick the k largest
  * (ties: lower expert index first; output ordered by descending value, then ascending index;
  * NaN ranks above +inf), and softmax over the k selected values in fp32

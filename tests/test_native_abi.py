@@ -26,6 +26,7 @@ def test_header_declares_the_expected_entry_points():
     for required in [
         "xma_continuous_count",
         "xma_route_build",
+        "xma_route_build_static",
         "xma_offsets_from_sorted",
         "xma_topk_softmax",
         "xma_topk_softmax_bwd",

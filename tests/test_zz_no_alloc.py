@@ -1,0 +1,84 @@
+"""xma_route_build_static, the routing entry point that allocates nothing: called through the C ABI, its four
+outputs must equal xma_route_build's bit for bit, on two calls in a row of which the second is smaller (the
+built-in working memory keeps the first call's contents), and sizes beyond the built-in memory are rejected."""
+
+import pytest
+import torch
+
+from flash_model_architectures_amd import _native
+
+pytestmark = pytest.mark.gpu
+
+
+def _outputs(n, E, index_dtype):
+    dev = "cuda"
+    return (
+        torch.full((E,), 0xFFFFFFFF, dtype=torch.uint32, device=dev),
+        torch.full((E + 1,), -7, dtype=torch.int32, device=dev),
+        torch.full((n,), -7, dtype=index_dtype, device=dev),
+        torch.full((n,), -7, dtype=index_dtype, device=dev),
+    )
+
+
+def _route_with_workspace(ids, E, index_dtype):
+    lib = _native.load()
+    n = ids.numel()
+    counts, offsets, sorted_ids, perm = _outputs(n, E, index_dtype)
+    ws_bytes = lib.xma_route_workspace_bytes(n, E)
+    workspace = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=ids.device)
+    _native.call(
+        "xma_route_build", ids.data_ptr(), int(ids.dtype == torch.int64), n, E, counts.data_ptr(), offsets.data_ptr(),
+        sorted_ids.data_ptr(), perm.data_ptr(), int(index_dtype == torch.int64), workspace.data_ptr(), workspace.numel(),
+        _native.stream(),
+    )  # fmt: skip
+    return counts, offsets, sorted_ids, perm
+
+
+def _route_static(ids, E, index_dtype):
+    n = ids.numel()
+    counts, offsets, sorted_ids, perm = _outputs(n, E, index_dtype)
+    _native.call(
+        "xma_route_build_static", ids.data_ptr(), int(ids.dtype == torch.int64), n, E, counts.data_ptr(),
+        offsets.data_ptr(), sorted_ids.data_ptr(), perm.data_ptr(), int(index_dtype == torch.int64), _native.stream(),
+    )  # fmt: skip
+    return counts, offsets, sorted_ids, perm
+
+
+def _same(got, want, what):
+    for g, w, name in zip(got, want, ("counts", "offsets", "sorted ids", "permutation")):
+        assert torch.equal(g.cpu().to(torch.int64), w.cpu().to(torch.int64)), f"{what}: {name} differ"
+
+
+def test_static_route_build_matches_route_build_on_two_calls_in_a_row():
+    g = torch.Generator().manual_seed(11)
+    # first call: the skewed-routing shape (131072 routed rows, 128 experts, some of them empty), int64 in and out
+    big = torch.randint(0, 128, (131072,), generator=g, dtype=torch.int64)
+    big[big % 9 == 4] = 1
+    big = big.cuda()
+    _same(_route_static(big, 128, torch.int64), _route_with_workspace(big, 128, torch.int64), "first call")
+    # second call, smaller, other types and expert count: nothing of the first call's histograms may leak in
+    small = torch.randint(0, 8, (3001,), generator=g, dtype=torch.int32).cuda()
+    _same(_route_static(small, 8, torch.int32), _route_with_workspace(small, 8, torch.int32), "second call")
+    # and the big one again after the small one
+    _same(_route_static(big, 128, torch.int64), _route_with_workspace(big, 128, torch.int64), "third call")
+    torch.cuda.synchronize()
+
+
+def test_static_route_build_edges_and_limit():
+    lib = _native.load()
+    # empty input: zero counts and offsets, as xma_route_build
+    empty = torch.empty(0, dtype=torch.int64, device="cuda")
+    counts, offsets, _, _ = _route_static(empty, 4, torch.int64)
+    assert counts.tolist() == [0] * 4 and offsets.tolist() == [0] * 5
+    # the largest case the built-in memory covers: ceil(n / 1024) * E * 4 bytes == the limit
+    limit = lib.xma_route_build_static_max_bytes()
+    assert limit == 1 << 20
+    n, E = 1 << 20, 256
+    assert lib.xma_route_workspace_bytes(n, E) == limit
+    ids = torch.randint(0, E, (n,), dtype=torch.int32, device="cuda")
+    _same(_route_static(ids, E, torch.int32), _route_with_workspace(ids, E, torch.int32), "limit case")
+    # one chunk more is rejected on the host, before any launch, with a message that names the way out
+    ids = torch.zeros(n + 1, dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="xma_route_build with a caller-owned workspace"):
+        _route_static(ids, E, torch.int32)
+    torch.cuda.synchronize()
