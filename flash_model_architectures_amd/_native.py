@@ -20,7 +20,7 @@ _lib: ctypes.CDLL | None = None
 DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 GEMM_TN, GEMM_NN, GEMM_MT = 0, 1, 2
-EPI_NONE, EPI_SWIGLU, EPI_SWIGLU_BWD = 0, 1, 2
+EPI_NONE, EPI_SWIGLU, EPI_SWIGLU_BWD, EPI_GLU, EPI_GLU_BWD, EPI_GELU_TANH, EPI_GELU_TANH_BWD = 0, 1, 2, 3, 4, 5, 6
 
 
 class GroupedGemmArgs(ctypes.Structure):
@@ -51,6 +51,8 @@ class GroupedGemmArgs(ctypes.Structure):
         ("in_fan_out", c_int32),
         ("workspace", c_void_p),
         ("workspace_bytes", c_int64),
+        ("bias", c_void_p),
+        ("ld_bias", c_int64),
     ]
 
 

@@ -134,6 +134,52 @@ __device__ __forceinline__ float sigmoid_fast(float x) {
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
 }
 
+// The activations the grouped GEMM epilogues fuse, forward and backward, on fp32 values.  FAST selects the hardware
+// exp2 / reciprocal (a few ulp in fp32) for results that are rounded to a 16-bit type anyway.
+enum Activation { ACT_NONE = 0, ACT_SWIGLU = 1, ACT_GLU = 2, ACT_GELU_TANH = 3 };
+
+template <bool FAST>
+__device__ __forceinline__ float sigmoid_any(float x) {
+    if constexpr (FAST) return sigmoid_fast(x);
+    else return sigmoid_f32(x);
+}
+
+// act(a, b) of the two halves of a gated pre-activation: SwiGLU a * b * sigmoid(b) (a = up, b = gate,
+// xma/functional/swiglu/__init__.py:34-43); GLU a * sigmoid(b) (torch.nn.GLU)
+template <bool FAST>
+__device__ __forceinline__ float gated_forward(int act, float a, float b) {
+    const float s = sigmoid_any<FAST>(b);
+    return act == ACT_SWIGLU ? a * (b * s) : a * s;
+}
+// gradients with respect to a and b for an upstream gradient d
+template <bool FAST>
+__device__ __forceinline__ void gated_backward(int act, float a, float b, float d, float& da, float& db) {
+    const float s = sigmoid_any<FAST>(b);
+    if (act == ACT_SWIGLU) {  // xma/functional/swiglu/triton_implementation/backward.py:45-56
+        const float t = b * s;
+        da = d * t;
+        db = d * a * (s + t * (1.0f - s));
+    } else {
+        da = d * s;
+        db = d * a * (s * (1.0f - s));
+    }
+}
+
+// tanh-approximated GELU and its derivative; tanh(u) = 2 sigmoid(2u) - 1
+template <bool FAST>
+__device__ __forceinline__ float gelu_tanh_forward(float x) {
+    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    return x * sigmoid_any<FAST>(2.0f * u);  // 0.5 x (1 + tanh u)
+}
+template <bool FAST>
+__device__ __forceinline__ float gelu_tanh_backward(float x, float d) {
+    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    const float s = sigmoid_any<FAST>(2.0f * u);  // (1 + tanh u) / 2
+    const float du = 0.7978845608028654f * (1.0f + 3.0f * 0.044715f * x * x);
+    // d/dx [x s(2u)] = s + x * 2 s (1 - s) du
+    return d * (s + 2.0f * x * s * (1.0f - s) * du);
+}
+
 // ---- wave64 primitives ------------------------------------------------------------------------
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (kWaveSize - 1)); }
 

@@ -169,7 +169,7 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
     constexpr int C_ROW_BYTES = BN * (int)sizeof(T) + 16;
     // column tile width in units of output columns: the SwiGLU epilogue packs BN/2 `up` and BN/2
     // `gate` columns into one tile
-    constexpr int BN_OUT = EPI == XMA_EPI_SWIGLU ? BN / 2 : BN;
+    constexpr int BN_OUT = EPI == EPI_PAIRED ? BN / 2 : BN;
     static_assert(BK * sizeof(T) == kLdsRowBytes, "LDS rows are 128 bytes");
 
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
     if constexpr (!B_TRANS) {
         b_direct.init(tid, [&](int r) -> const T* {
             int64_t n;
-            if constexpr (EPI == XMA_EPI_SWIGLU) {
+            if constexpr (EPI == EPI_PAIRED) {
                 const int64_t half = P.n / 2;
                 const int64_t j = n0 + (r % BN_OUT);
                 if (j >= half) return nullptr;
@@ -374,8 +374,28 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
             for (int g = 0; g < 4; ++g) {
                 const int col = wn0 + ni * 32 + 8 * g + 4 * frag_half;
                 char* dst = lds + row * C_ROW_BYTES + col * (int)sizeof(T);
-                const float f[4] = {acc[mi][ni][4 * g], acc[mi][ni][4 * g + 1], acc[mi][ni][4 * g + 2],
-                                    acc[mi][ni][4 * g + 3]};
+                float f[4] = {acc[mi][ni][4 * g], acc[mi][ni][4 * g + 1], acc[mi][ni][4 * g + 2], acc[mi][ni][4 * g + 3]};
+                if constexpr (KIND == XMA_GEMM_TN) {
+                    // the expert's bias, added to the fp32 sums before they are rounded; tile column `col` is
+                    // weight row n0 + col, or for a gated tile n0 + col (first half) and N/2 + n0 + col - BN_OUT
+                    if (P.bias != nullptr) {
+                        int64_t n;
+                        bool exists;
+                        if constexpr (EPI == EPI_PAIRED) {
+                            const int64_t half_n = P.n / 2;
+                            n = n0 + (col % BN_OUT) + (col >= BN_OUT ? half_n : 0);
+                            exists = n0 + (col % BN_OUT) < half_n;
+                        } else {
+                            n = n0 + col;
+                            exists = n < P.n;
+                        }
+                        if (exists) {
+                            const T* b = reinterpret_cast<const T*>(P.bias) + (int64_t)expert * P.ld_bias + n;
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) f[q] += Elem<T>::load(b + q);
+                        }
+                    }
+                }
                 if constexpr (sizeof(T) == 4) {
                     *reinterpret_cast<uint4*>(dst) = Elem<float>::pack(f);
                 } else {
@@ -402,10 +422,22 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
             const int64_t p = m_begin + r;
             if (p >= m_end) break;
             const int64_t orow = P.out_index ? load_index(P.out_index, P.idx_is_i64, p) : p;
-            if constexpr (EPI == XMA_EPI_NONE) {
+            if constexpr (EPI == EPI_PLAIN) {
                 const int64_t n = n0 + cc * PV;
-                if (n < P.n) *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = *reinterpret_cast<const uint4*>(src + cc * 16);
-            } else if constexpr (EPI == XMA_EPI_SWIGLU) {
+                if (n < P.n) {
+                    const uint4 v = *reinterpret_cast<const uint4*>(src + cc * 16);
+                    if (KIND == XMA_GEMM_TN && P.act == ACT_GELU_TANH) {
+                        if (P.aux) *reinterpret_cast<uint4*>(reinterpret_cast<T*>(P.aux) + p * P.ld_aux + n) = v;
+                        float h[PV], o[PV];
+                        Elem<T>::unpack(v, h);
+#pragma unroll
+                        for (int q = 0; q < PV; ++q) o[q] = gelu_tanh_forward<false>(h[q]);
+                        *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = Elem<T>::pack(o);
+                    } else {
+                        *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = v;
+                    }
+                }
+            } else if constexpr (EPI == EPI_PAIRED) {
                 constexpr int HALF_CHUNKS = C_CHUNKS / 2;
                 const int64_t half = P.n / 2;
                 const int64_t j = n0 + (cc % HALF_CHUNKS) * PV;
@@ -420,26 +452,28 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
                         Elem<T>::unpack(*reinterpret_cast<const uint4*>(src + cc * 16), u);
                         Elem<T>::unpack(*reinterpret_cast<const uint4*>(src + (cc + HALF_CHUNKS) * 16), g);
 #pragma unroll
-                        for (int q = 0; q < PV; ++q) o[q] = u[q] * (g[q] * sigmoid_f32(g[q]));
+                        for (int q = 0; q < PV; ++q) o[q] = gated_forward<false>(P.act, u[q], g[q]);
                         *reinterpret_cast<uint4*>(C + orow * P.ldc + j) = Elem<T>::pack(o);
                     }
                 }
-            } else {  // XMA_EPI_SWIGLU_BWD
+            } else {  // EPI_BACKWARD: the product is the activation's upstream gradient
                 const int64_t n = n0 + cc * PV;
                 if (n < P.n) {
                     const T* h = reinterpret_cast<const T*>(P.aux) + p * P.ld_aux;
                     float u[PV], g[PV], d[PV], du[PV], dg[PV];
                     Elem<T>::unpack(load16(h + n), u);
-                    Elem<T>::unpack(load16(h + P.n + n), g);
                     Elem<T>::unpack(*reinterpret_cast<const uint4*>(src + cc * 16), d);
+                    if (P.act == ACT_GELU_TANH) {
 #pragma unroll
-                    for (int q = 0; q < PV; ++q) {
-                        const float sg = sigmoid_f32(g[q]);
-                        dg[q] = d[q] * u[q] * (sg + g[q] * sg * (1.0f - sg));
-                        du[q] = d[q] * g[q] * sg;
+                        for (int q = 0; q < PV; ++q) du[q] = gelu_tanh_backward<false>(u[q], d[q]);
+                        *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = Elem<T>::pack(du);
+                    } else {
+                        Elem<T>::unpack(load16(h + P.n + n), g);
+#pragma unroll
+                        for (int q = 0; q < PV; ++q) gated_backward<false>(P.act, u[q], g[q], d[q], du[q], dg[q]);
+                        *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = Elem<T>::pack(du);
+                        *reinterpret_cast<uint4*>(C + orow * P.ldc + P.n + n) = Elem<T>::pack(dg);
                     }
-                    *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = Elem<T>::pack(du);
-                    *reinterpret_cast<uint4*>(C + orow * P.ldc + P.n + n) = Elem<T>::pack(dg);
                 }
             }
         }
@@ -473,8 +507,8 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
         P.tile_expert = ws + 4;
         P.tile_row0 = ws + 4 + rt;
         P.row_tiles_max = (int32_t)rt;
-        const int bn_out = EPI == XMA_EPI_SWIGLU ? Cfg::BN / 2 : Cfg::BN;
-        const int64_t n_out = EPI == XMA_EPI_SWIGLU ? a.n / 2 : a.n;
+        const int bn_out = EPI == EPI_PAIRED ? Cfg::BN / 2 : Cfg::BN;
+        const int64_t n_out = EPI == EPI_PAIRED ? a.n / 2 : a.n;
         P.col_tiles = (int32_t)ceil_div(n_out, bn_out);
         grid = grid_for_tiles(rt, P.col_tiles);
         hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(1024), 0, stream, a.expert_offsets, a.num_experts,
@@ -502,6 +536,10 @@ void fill_params(const xma_grouped_gemm_args& a, GemmParams& P) {
     P.aux = a.aux;
     P.offsets = a.expert_offsets;
     P.expert_order = nullptr;
+    P.bias = a.bias;
+    P.ld_bias = a.ld_bias;
+    int shape = 0;
+    split_epilogue(a.epilogue, shape, P.act);
     P.in_index = a.in_index;
     P.out_index = a.out_index;
     P.lda = a.lda;
@@ -524,15 +562,17 @@ void fill_params(const xma_grouped_gemm_args& a, GemmParams& P) {
 
 template <typename T>
 static int dispatch_kind(const xma_grouped_gemm_args& a, hipStream_t stream) {
+    int shape = EPI_PLAIN, act = ACT_NONE;
+    split_epilogue(a.epilogue, shape, act);
     switch (a.kind) {
         case XMA_GEMM_TN:
-            if (a.epilogue == XMA_EPI_SWIGLU) return launch<T, XMA_GEMM_TN, XMA_EPI_SWIGLU>(a, stream);
-            return launch<T, XMA_GEMM_TN, XMA_EPI_NONE>(a, stream);
+            if (shape == EPI_PAIRED) return launch<T, XMA_GEMM_TN, EPI_PAIRED>(a, stream);
+            return launch<T, XMA_GEMM_TN, EPI_PLAIN>(a, stream);
         case XMA_GEMM_NN:
-            if (a.epilogue == XMA_EPI_SWIGLU_BWD) return launch<T, XMA_GEMM_NN, XMA_EPI_SWIGLU_BWD>(a, stream);
-            return launch<T, XMA_GEMM_NN, XMA_EPI_NONE>(a, stream);
+            if (shape == EPI_BACKWARD) return launch<T, XMA_GEMM_NN, EPI_BACKWARD>(a, stream);
+            return launch<T, XMA_GEMM_NN, EPI_PLAIN>(a, stream);
         default:
-            return launch<T, XMA_GEMM_MT, XMA_EPI_NONE>(a, stream);
+            return launch<T, XMA_GEMM_MT, EPI_PLAIN>(a, stream);
     }
 }
 
@@ -572,7 +612,7 @@ int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
                 "xma_grouped_gemm: operands must be 16-byte aligned");
     const bool mt = a.kind == XMA_GEMM_MT;
     if (mt) {
-        XMA_REQUIRE(a.epilogue == XMA_EPI_NONE, "xma_grouped_gemm: MT takes no epilogue");
+        XMA_REQUIRE(a.epilogue == XMA_EPI_NONE && a.bias == nullptr, "xma_grouped_gemm: MT takes no epilogue and no bias");
         XMA_REQUIRE(a.lda >= a.n && a.ldb >= a.k && a.ldc >= a.k, "xma_grouped_gemm: MT row strides too small");
         XMA_REQUIRE(a.out_index == nullptr, "xma_grouped_gemm: MT takes no out_index");
         XMA_REQUIRE(a.workspace == nullptr || a.workspace_bytes >= expert_order_bytes(a.num_experts),
@@ -580,22 +620,33 @@ int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
                     (long long)expert_order_bytes(a.num_experts));
         if (a.n == 0 || a.k == 0) return 0;
     } else {
-        XMA_REQUIRE(a.epilogue == XMA_EPI_NONE || (a.kind == XMA_GEMM_TN && a.epilogue == XMA_EPI_SWIGLU) ||
-                        (a.kind == XMA_GEMM_NN && a.epilogue == XMA_EPI_SWIGLU_BWD),
+        int shape = EPI_PLAIN, act = ACT_NONE;
+        split_epilogue(a.epilogue, shape, act);
+        const bool forward_epi = a.epilogue == XMA_EPI_SWIGLU || a.epilogue == XMA_EPI_GLU || a.epilogue == XMA_EPI_GELU_TANH;
+        const bool backward_epi =
+            a.epilogue == XMA_EPI_SWIGLU_BWD || a.epilogue == XMA_EPI_GLU_BWD || a.epilogue == XMA_EPI_GELU_TANH_BWD;
+        XMA_REQUIRE(a.epilogue == XMA_EPI_NONE || (a.kind == XMA_GEMM_TN && forward_epi) ||
+                        (a.kind == XMA_GEMM_NN && backward_epi),
                     "xma_grouped_gemm: epilogue %d not available for kind %d", a.epilogue, a.kind);
         XMA_REQUIRE(a.lda >= a.k, "xma_grouped_gemm: lda too small");
         XMA_REQUIRE(a.ldb >= (a.kind == XMA_GEMM_TN ? a.k : a.n), "xma_grouped_gemm: ldb too small");
-        if (a.epilogue == XMA_EPI_SWIGLU) {
-            XMA_REQUIRE(a.n % (2 * pv) == 0, "xma_grouped_gemm: SwiGLU epilogue needs n %% %d == 0", 2 * pv);
+        if (shape == EPI_PAIRED) {
+            XMA_REQUIRE(a.n % (2 * pv) == 0, "xma_grouped_gemm: gated epilogue needs n %% %d == 0", 2 * pv);
             XMA_REQUIRE(a.ldc >= a.n / 2, "xma_grouped_gemm: ldc too small");
             XMA_REQUIRE(a.aux == nullptr || a.ld_aux >= a.n, "xma_grouped_gemm: ld_aux too small");
-        } else if (a.epilogue == XMA_EPI_SWIGLU_BWD) {
-            XMA_REQUIRE(a.aux != nullptr && a.ld_aux >= 2 * a.n && a.ldc >= 2 * a.n,
-                        "xma_grouped_gemm: SwiGLU backward epilogue needs aux/ldc of 2n columns");
-            XMA_REQUIRE(a.out_index == nullptr, "xma_grouped_gemm: SwiGLU backward epilogue writes grouped rows");
+        } else if (shape == EPI_BACKWARD) {
+            const int64_t saved = act == ACT_GELU_TANH ? a.n : 2 * a.n;  // columns of the saved pre-activation
+            XMA_REQUIRE(a.aux != nullptr && a.ld_aux >= saved && a.ldc >= saved,
+                        "xma_grouped_gemm: activation backward epilogue needs aux/ldc of %lld columns", (long long)saved);
+            XMA_REQUIRE(a.out_index == nullptr, "xma_grouped_gemm: activation backward epilogue writes grouped rows");
         } else {
             XMA_REQUIRE(a.ldc >= a.n, "xma_grouped_gemm: ldc too small");
+            XMA_REQUIRE(act == ACT_NONE || a.aux == nullptr || a.ld_aux >= a.n, "xma_grouped_gemm: ld_aux too small");
+            XMA_REQUIRE(act == ACT_NONE || a.out_index == nullptr || a.aux == nullptr,
+                        "xma_grouped_gemm: the pre-activation is kept for grouped outputs only");
         }
+        XMA_REQUIRE(a.bias == nullptr || (a.kind == XMA_GEMM_TN && a.ld_bias >= a.n && a.ld_bias % pv == 0 && aligned16(a.bias)),
+                    "xma_grouped_gemm: bias needs a forward (TN) kind, ld_bias >= n and 16-byte aligned rows");
         if (a.rows == 0 || a.n == 0) return 0;
         XMA_REQUIRE(a.workspace != nullptr &&
                         a.workspace_bytes >= xma_grouped_gemm_workspace_bytes(a.num_experts, a.rows),

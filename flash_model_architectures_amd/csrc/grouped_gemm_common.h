@@ -38,7 +38,29 @@ struct GemmParams {
     // MT: experts in descending order of their row counts, one record {expert, first row, end row, 0} per slot;
     // nullptr: slot e is expert e
     const int32_t* expert_order;
+    // fused activation of the epilogue (enum Activation) and the optional per-expert bias of the forward kinds
+    const void* bias;
+    int64_t ld_bias;
+    int32_t act;
 };
+
+// The kernels are instantiated for three epilogue shapes; the activation inside a shape is a run-time value
+// (GemmParams::act), so SwiGLU and GLU, or the two backward forms, share one instantiation.
+//   EPI_PLAIN     store the product (optionally through tanh-GELU, keeping the pre-activation)
+//   EPI_PAIRED    TN: tile columns [0, 128) and [128, 256) are the two halves of a gated pre-activation
+//   EPI_BACKWARD  NN: the product is the activation's upstream gradient; the saved pre-activation is read back
+constexpr int EPI_PLAIN = 0, EPI_PAIRED = 1, EPI_BACKWARD = 2;
+inline void split_epilogue(int epilogue, int& shape, int& act) {
+    switch (epilogue) {
+        case XMA_EPI_SWIGLU: shape = EPI_PAIRED; act = ACT_SWIGLU; break;
+        case XMA_EPI_GLU: shape = EPI_PAIRED; act = ACT_GLU; break;
+        case XMA_EPI_SWIGLU_BWD: shape = EPI_BACKWARD; act = ACT_SWIGLU; break;
+        case XMA_EPI_GLU_BWD: shape = EPI_BACKWARD; act = ACT_GLU; break;
+        case XMA_EPI_GELU_TANH: shape = EPI_PLAIN; act = ACT_GELU_TANH; break;
+        case XMA_EPI_GELU_TANH_BWD: shape = EPI_BACKWARD; act = ACT_GELU_TANH; break;
+        default: shape = EPI_PLAIN; act = ACT_NONE; break;
+    }
+}
 
 // At most kSplitSlots (tile, part) pairs exist at a time: the split tiles are those of one round of the device.
 constexpr int kSplitSlots = 256;

@@ -291,7 +291,7 @@ struct Kernel {
     using G = Geometry<BK>;
     static constexpr bool A_STRIDED = KIND == XMA_GEMM_MT;
     static constexpr bool B_STRIDED = KIND != XMA_GEMM_TN;
-    static constexpr int BN_OUT = EPI == XMA_EPI_SWIGLU ? BN / 2 : BN;
+    static constexpr int BN_OUT = EPI == EPI_PAIRED ? BN / 2 : BN;
 
     OperandLoads<T, BK, A_STRIDED ? PLAN_STRIDED : PLAN_ROWS> la;
     OperandLoads<T, BK, B_STRIDED ? PLAN_STRIDED : PLAN_UNIFORM> lb;
@@ -540,7 +540,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             });
         const T* W = B + (int64_t)expert * P.b_expert_stride;
         if constexpr (KIND == XMA_GEMM_TN) {
-            if constexpr (EPI == XMA_EPI_SWIGLU) {
+            if constexpr (EPI == EPI_PAIRED) {
                 // tile rows 0..127: weight rows n0 + r (up half); rows 128..255: P.n / 2 + n0 + r - 128 (gate half)
                 const int64_t half = P.n / 2;
                 k.lb.setup_uniform(k.wave, k.lane, W + n0 * P.ldb, P.ldb, (half - BN_OUT) * P.ldb,
@@ -671,7 +671,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                     orow[mi][it] = p < m_end ? orow[mi][it] : -1;
                 }
         };
-        if (EPI == XMA_EPI_SWIGLU_BWD || P.out_index == nullptr)  // that epilogue only writes grouped rows
+        if (EPI == EPI_BACKWARD || P.out_index == nullptr)  // that epilogue only writes grouped rows
             fill([&](int64_t p) { return (int32_t)p; });
         else if (P.idx_is_i64)
             fill([&](int64_t p) { return (int32_t)reinterpret_cast<const int64_t*>(P.out_index)[p]; });
@@ -679,19 +679,21 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             fill([&](int64_t p) { return reinterpret_cast<const int32_t*>(P.out_index)[p]; });
     }
 
-    // SwiGLU backward: the saved pre-activation chunks (up, gate) of the rows of slab mi, double-buffered so
-    // that slab mi+1 is on its way from HBM while slab mi is processed
-    constexpr bool SWBWD = EPI == XMA_EPI_SWIGLU_BWD;
+    // Activation backward: the saved pre-activation chunks (the two halves of a gated one; tanh-GELU has a single
+    // half, fetched twice) of the rows of slab mi, double-buffered so that slab mi+1 is on its way from HBM while
+    // slab mi is processed
+    constexpr bool SWBWD = EPI == EPI_BACKWARD;
     u32x4_t hu[SWBWD ? 2 : 1][IT], hg[SWBWD ? 2 : 1][IT];
     auto load_saved = [&](int mi, u32x4_t (&up)[IT], u32x4_t (&gate)[IT]) {
         // branch-free: rows / columns outside the tile's part of the operand re-read a valid chunk
         const int64_t n = n0 + cc * PV < P.n ? n0 + cc * PV : 0;
+        const int64_t second_half = P.act == ACT_GELU_TANH ? 0 : P.n;
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
             const int64_t p = m_begin + tile_row(mi, buffer_row(it));
             const T* h = reinterpret_cast<const T*>(P.aux) + (p < m_end ? p : m_end - 1) * P.ld_aux;
             up[it] = *reinterpret_cast<const u32x4_t*>(h + n);
-            gate[it] = *reinterpret_cast<const u32x4_t*>(h + P.n + n);
+            gate[it] = *reinterpret_cast<const u32x4_t*>(h + second_half + n);
         }
     };
     if constexpr (SWBWD) load_saved(0, hu[0], hg[0]);
@@ -702,15 +704,52 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         const int wn0 = (k.wave % WAVES_N) * WN;
         const int br = (k.wave / WAVES_N) * 32 + (etid & 31);
         const int half = (etid >> 5) & 1;
+        // Forward kinds: the expert's bias row, added to the fp32 sums before they are rounded.  Tile column c is
+        // weight row n0 + c, or for a gated tile n0 + c (c < 128) and N/2 + n0 + c - 128 (c >= 128).
+        float bias[KIND == XMA_GEMM_TN ? NI : 1][KIND == XMA_GEMM_TN ? 4 : 1][KIND == XMA_GEMM_TN ? 4 : 1];
+        bool with_bias = false;
+        if constexpr (KIND == XMA_GEMM_TN) {
+            with_bias = P.bias != nullptr;
+            if (with_bias) {
+                const T* row = reinterpret_cast<const T*>(P.bias) + (int64_t)expert * P.ld_bias;
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int c = wn0 + ni * 32 + 8 * g + 4 * half;
+                        int64_t n;
+                        bool exists;
+                        if constexpr (EPI == EPI_PAIRED) {
+                            const int64_t half_n = P.n / 2;
+                            n = n0 + (c % BN_OUT) + (c >= BN_OUT ? half_n : 0);
+                            exists = n0 + (c % BN_OUT) < half_n;
+                        } else {
+                            n = n0 + c;
+                            exists = n < P.n;
+                        }
+                        const uint2 raw = *reinterpret_cast<const uint2*>(row + (exists ? n : 0));
+                        float v[8];
+                        Elem<T>::unpack(make_uint4(raw.x, raw.y, 0u, 0u), v);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) bias[ni][g][q] = exists ? v[q] : 0.0f;
+                    }
+            }
+        }
         auto write_rows = [&](char* buf, const f32x16_t (&a)[NI]) {
 #pragma unroll
             for (int ni = 0; ni < NI; ++ni) {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const int chunk = ((wn0 + ni * 32 + 8 * g) >> 3) ^ (br & 31);
+                    float v[4] = {a[ni][4 * g], a[ni][4 * g + 1], a[ni][4 * g + 2], a[ni][4 * g + 3]};
+                    if constexpr (KIND == XMA_GEMM_TN) {
+                        if (with_bias) {
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) v[q] += bias[ni][g][q];
+                        }
+                    }
                     *reinterpret_cast<uint2*>(buf + br * (BN * 2) + (chunk << 4) + half * 8) =
-                        make_uint2(Elem<T>::pack2(a[ni][4 * g], a[ni][4 * g + 1]),
-                                   Elem<T>::pack2(a[ni][4 * g + 2], a[ni][4 * g + 3]));
+                        make_uint2(Elem<T>::pack2(v[0], v[1]), Elem<T>::pack2(v[2], v[3]));
                 }
             }
         };
@@ -747,15 +786,30 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                 // operand panels of the running tiles out of the caches (1-2 % on this kind)
                 if (i < P.n && j < P.k) __builtin_nontemporal_store(v[it], reinterpret_cast<u32x4_t*>(out + i * P.ldc));
             }
-        } else if constexpr (EPI == XMA_EPI_NONE) {
+        } else if constexpr (EPI == EPI_PLAIN) {
             const int64_t n = n0 + cc * PV;
             u32x4_t v[IT];
             read_own_chunks(v);
+            if (KIND == XMA_GEMM_TN && P.act == ACT_GELU_TANH) {
+                // tanh-GELU of the product; the rounded product itself is kept as the pre-activation
 #pragma unroll
-            for (int it = 0; it < IT; ++it)
-                if (out_row[it] >= 0 && n < P.n)
-                    *reinterpret_cast<u32x4_t*>(C + (int64_t)out_row[it] * P.ldc + n) = v[it];
-        } else if constexpr (EPI == XMA_EPI_SWIGLU) {
+                for (int it = 0; it < IT; ++it) {
+                    if (out_row[it] < 0 || n >= P.n) continue;
+                    const int64_t p = m_begin + tile_row(mi, buffer_row(it));
+                    if (P.aux) *reinterpret_cast<u32x4_t*>(reinterpret_cast<T*>(P.aux) + p * P.ld_aux + n) = v[it];
+                    float h[PV], o[PV];
+                    Elem<T>::unpack(to_uint4(v[it]), h);
+#pragma unroll
+                    for (int q = 0; q < PV; ++q) o[q] = gelu_tanh_forward<true>(h[q]);
+                    *reinterpret_cast<uint4*>(C + (int64_t)out_row[it] * P.ldc + n) = Elem<T>::pack(o);
+                }
+            } else {
+#pragma unroll
+                for (int it = 0; it < IT; ++it)
+                    if (out_row[it] >= 0 && n < P.n)
+                        *reinterpret_cast<u32x4_t*>(C + (int64_t)out_row[it] * P.ldc + n) = v[it];
+            }
+        } else if constexpr (EPI == EPI_PAIRED) {
             // The slab row holds 16 chunks of the up half, then the 16 matching chunks of the gate half.  Thread
             // cc handles chunk pair cc % 16 on every other owned row (even `it` for cc < 16, odd otherwise), so
             // that every lane computes.
@@ -793,7 +847,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                 Elem<T>::unpack(to_uint4(up), u);
                 Elem<T>::unpack(to_uint4(gate), g);
 #pragma unroll
-                for (int q = 0; q < PV; ++q) o[q] = u[q] * (g[q] * sigmoid_fast(g[q]));
+                for (int q = 0; q < PV; ++q) o[q] = gated_forward<true>(P.act, u[q], g[q]);
                 *reinterpret_cast<uint4*>(C + (int64_t)row_out * P.ldc + j) = Elem<T>::pack(o);
             }
         } else {  // XMA_EPI_SWIGLU_BWD
@@ -808,16 +862,17 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                 Elem<T>::unpack(to_uint4(hu[mi & 1][it]), u);
                 Elem<T>::unpack(to_uint4(hg[mi & 1][it]), g);
                 Elem<T>::unpack(to_uint4(dv[it]), d);
-#pragma unroll
-                for (int q = 0; q < PV; ++q) {
-                    const float sg = sigmoid_fast(g[q]);
-                    const float t = g[q] * sg;
-                    du[q] = d[q] * t;
-                    dg[q] = d[q] * u[q] * (sg + t * (1.0f - sg));
-                }
                 T* out = C + (int64_t)out_row[it] * P.ldc;
-                *reinterpret_cast<uint4*>(out + n) = Elem<T>::pack(du);
-                *reinterpret_cast<uint4*>(out + P.n + n) = Elem<T>::pack(dg);
+                if (P.act == ACT_GELU_TANH) {
+#pragma unroll
+                    for (int q = 0; q < PV; ++q) du[q] = gelu_tanh_backward<true>(u[q], d[q]);
+                    *reinterpret_cast<uint4*>(out + n) = Elem<T>::pack(du);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < PV; ++q) gated_backward<true>(P.act, u[q], g[q], d[q], du[q], dg[q]);
+                    *reinterpret_cast<uint4*>(out + n) = Elem<T>::pack(du);
+                    *reinterpret_cast<uint4*>(out + P.n + n) = Elem<T>::pack(dg);
+                }
             }
         }
     };
@@ -867,8 +922,8 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
         P.split_counters = reinterpret_cast<int32_t*>(split);
         P.split_partials = reinterpret_cast<float*>(split + kSplitSlots * sizeof(int32_t));
         P.num_cu = compute_units();
-        const int bn_out = EPI == XMA_EPI_SWIGLU ? BN / 2 : BN;
-        const int64_t n_out = EPI == XMA_EPI_SWIGLU ? a.n / 2 : a.n;
+        const int bn_out = EPI == EPI_PAIRED ? BN / 2 : BN;
+        const int64_t n_out = EPI == EPI_PAIRED ? a.n / 2 : a.n;
         P.col_tiles = (int32_t)ceil_div(n_out, bn_out);
         grid = grid_for_work(rt * P.col_tiles);
         hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(1024), 0, stream, a.expert_offsets, a.num_experts, BM,
@@ -884,15 +939,17 @@ static int dispatch(const xma_grouped_gemm_args& a, hipStream_t stream) {
     using PipeTN = Ring64x5;
     using PipeNN = Ring64x5;
     using PipeMT = Ring64x5;
+    int shape = EPI_PLAIN, act = ACT_NONE;
+    split_epilogue(a.epilogue, shape, act);
     switch (a.kind) {
         case XMA_GEMM_TN:
-            if (a.epilogue == XMA_EPI_SWIGLU) return launch<T, XMA_GEMM_TN, XMA_EPI_SWIGLU, PipeTN>(a, stream);
-            return launch<T, XMA_GEMM_TN, XMA_EPI_NONE, PipeTN>(a, stream);
+            if (shape == EPI_PAIRED) return launch<T, XMA_GEMM_TN, EPI_PAIRED, PipeTN>(a, stream);
+            return launch<T, XMA_GEMM_TN, EPI_PLAIN, PipeTN>(a, stream);
         case XMA_GEMM_NN:
-            if (a.epilogue == XMA_EPI_SWIGLU_BWD) return launch<T, XMA_GEMM_NN, XMA_EPI_SWIGLU_BWD, PipeNN>(a, stream);
-            return launch<T, XMA_GEMM_NN, XMA_EPI_NONE, PipeNN>(a, stream);
+            if (shape == EPI_BACKWARD) return launch<T, XMA_GEMM_NN, EPI_BACKWARD, PipeNN>(a, stream);
+            return launch<T, XMA_GEMM_NN, EPI_PLAIN, PipeNN>(a, stream);
         default:
-            return launch<T, XMA_GEMM_MT, XMA_EPI_NONE, PipeMT>(a, stream);
+            return launch<T, XMA_GEMM_MT, EPI_PLAIN, PipeMT>(a, stream);
     }
 }
 

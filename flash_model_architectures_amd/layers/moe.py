@@ -4,9 +4,11 @@
 -> grouped up-projection -> activation -> grouped down-projection scattered back and combined with
 the routing weights.  Two expert pipelines exist:
 
-* `_SwigluExperts`: when the activation is this package's `swiglu_packed`, SwiGLU is fused into the
-  up-projection's epilogue and its backward into the down-projection's input-gradient epilogue.
-* `scattered_experts` (+ any activation callable): the general pipeline with the same call
+* `_FusedExperts`: when the activation is one the kernels know (this package's `swiglu_packed`, `torch.nn.GLU`
+  over the last dimension, tanh-approximated `torch.nn.GELU`), it is fused into the up-projection's epilogue
+  and its backward into the down-projection's input-gradient epilogue; expert biases are added to the fp32
+  products inside the two forward kernels.
+* `scattered_experts` (+ any other activation callable): the general pipeline with the same call
   structure as the reference's `_ScatteredExperts`
   (xma/layers/moe/triton_implementation/__init__.py:14-185).
 """
@@ -22,16 +24,15 @@ from ..accelerator import KernelBackend, resolve_backend
 from ..functional.routing import route_tokens, topk_softmax
 from ..functional.swiglu_packed import swiglu_packed
 from ..ops import (
-    add_expert_bias,
     exclusive_offsets,
     combine_topk,
-    down_projection_dgrad_swiglu,
+    down_projection_dgrad_fused,
     expert_colsum,
     gate_grad,
     group,
     group_bwd_W,
     scatter2scatter,
-    up_projection_swiglu,
+    up_projection_fused,
 )
 from ..utils import XMAModule
 
@@ -65,15 +66,8 @@ class _ScatteredExperts(torch.autograd.Function):
             FAN_OUT=k,
             x_grouped=grouped_in,
             y_grouped=grouped_out,
+            bias=bias,  # F.linear(x, W[e], bias[e]) of the reference's torch path (xma/layers/moe/__init__.py:103-106)
         )
-        if bias is not None:
-            # F.linear(x, W[e], bias[e]) of the reference's torch path (xma/layers/moe/__init__.py:103-106)
-            add_expert_bias(
-                y=expanded,
-                bias=bias,
-                sorted_expert_idxs=sorted_expert_idxs,
-                out_index=None if grouped_out else sorted_scattered_idxs,
-            )
         if gates is None:
             output, saved_expanded = expanded, None
         else:
@@ -187,19 +181,34 @@ def scattered_experts(
     )
 
 
-class _SwigluExperts(torch.autograd.Function):
-    """Both projections with SwiGLU fused; weights in their stored layouts [E, 2I, H] and [E, H, I]."""
+def fused_activation_name(activation: Callable, is_glu: bool) -> str | None:
+    """The kernels' name for an activation callable (a key of ops.FUSED_ACTIVATIONS), or None when the callable
+    is not one they fuse and the layer has to take the general pipeline."""
+
+    if activation is swiglu_packed and is_glu:
+        return "swiglu"
+    if isinstance(activation, nn.GLU) and activation.dim in (-1, 1) and is_glu:
+        return "glu"  # the projection output is 2-D, so dim 1 is the last dimension too
+    if isinstance(activation, nn.GELU) and activation.approximate == "tanh" and not is_glu:
+        return "gelu_tanh"
+    return None
+
+
+class _FusedExperts(torch.autograd.Function):
+    """Both projections with the activation (and the biases) fused; weights in their stored layouts
+    [E, 2I or I, H] and [E, H, I]."""
 
     @staticmethod
-    def forward(ctx, x, w_up, w_down, gates, sorted_scattered_idxs, expert_offsets):
+    def forward(ctx, x, w_up, w_down, gates, sorted_scattered_idxs, expert_offsets, b_up, b_down, activation):
         T, H = x.shape
-        E, I2, _ = w_up.shape
+        E, N, _ = w_up.shape
+        I = w_down.size(2)
         k = gates.size(1)
         M = T * k
         needs_grad = any(ctx.needs_input_grad)
-        preact = torch.empty(M, I2, device=x.device, dtype=x.dtype) if needs_grad else None
-        act = torch.empty(M, I2 // 2, device=x.device, dtype=x.dtype)
-        up_projection_swiglu(
+        preact = torch.empty(M, N, device=x.device, dtype=x.dtype) if needs_grad else None
+        act = torch.empty(M, I, device=x.device, dtype=x.dtype)
+        up_projection_fused(
             X=x,
             W=w_up,
             sorted_scattered_idxs=sorted_scattered_idxs,
@@ -207,6 +216,8 @@ class _SwigluExperts(torch.autograd.Function):
             act=act,
             preact=preact,
             FAN_OUT=k,
+            activation=activation,
+            bias=b_up,
         )
         expanded = torch.empty(M, H, device=x.device, dtype=x.dtype)
         scatter2scatter(
@@ -219,18 +230,21 @@ class _SwigluExperts(torch.autograd.Function):
             FAN_OUT=1,
             x_grouped=True,
             y_grouped=False,
+            bias=b_down,
         )
         y = torch.empty(T, H, device=x.device, dtype=x.dtype)
         combine_topk(expanded=expanded, out=y, k=k, gates=gates)
         if needs_grad:
             ctx.save_for_backward(x, w_up, w_down, gates, sorted_scattered_idxs, expert_offsets, preact, act, expanded)
+        ctx.activation = activation
+        ctx.has_bias = b_up is not None, b_down is not None
         return y
 
     @staticmethod
     def backward(ctx, grad_out):
         x, w_up, w_down, gates, idx, expert_offsets, preact, act, expanded = ctx.saved_tensors
         T, H = x.shape
-        E, I2, _ = w_up.shape
+        E = w_up.size(0)
         k = gates.size(1)
         M = T * k
         if not grad_out.is_contiguous():  # e.g. the expanded (stride 0) gradient of y.sum() or y.mean(0)
@@ -242,13 +256,28 @@ class _SwigluExperts(torch.autograd.Function):
         grouped_grad = torch.empty(M, H, device=x.device, dtype=x.dtype)
         group(A=grad_out, sorted_expert_idxs=idx, out=grouped_grad, coeff=gates.flatten(), fan_out=k)
 
+        d_b_down = None
+        if ctx.has_bias[1] and ctx.needs_input_grad[7]:
+            d_b_down = torch.empty(E, H, device=x.device, dtype=x.dtype)
+            expert_colsum(src=grouped_grad, expert_offsets=expert_offsets, out=d_b_down)
+
         d_w_down = torch.empty_like(w_down)
         group_bwd_W(DY=grouped_grad, X=act, expert_offsets=expert_offsets, DW=d_w_down.permute(0, 2, 1), E=E)
 
         d_preact = torch.empty_like(preact)
-        down_projection_dgrad_swiglu(
-            DY=grouped_grad, W=w_down, preact=preact, expert_offsets=expert_offsets, d_preact=d_preact
+        down_projection_dgrad_fused(
+            DY=grouped_grad,
+            W=w_down,
+            preact=preact,
+            expert_offsets=expert_offsets,
+            d_preact=d_preact,
+            activation=ctx.activation,
         )
+
+        d_b_up = None
+        if ctx.has_bias[0] and ctx.needs_input_grad[6]:
+            d_b_up = torch.empty(E, preact.size(1), device=x.device, dtype=x.dtype)
+            expert_colsum(src=d_preact, expert_offsets=expert_offsets, out=d_b_up)
 
         d_w_up = torch.empty_like(w_up)
         group_bwd_W(
@@ -275,7 +304,7 @@ class _SwigluExperts(torch.autograd.Function):
         )
         d_x = torch.empty_like(x, memory_format=torch.contiguous_format)
         combine_topk(expanded=d_expanded, out=d_x, k=k, gates=None)
-        return d_x, d_w_up, d_w_down, d_gates, None, None
+        return d_x, d_w_up, d_w_down, d_gates, None, None, d_b_up, d_b_down, None
 
 
 class Experts(XMAModule):
@@ -467,16 +496,19 @@ class MoE(XMAModule):
 
         routing = route_tokens(selected_experts, self.num_experts)
 
-        # biases (torch path only in the reference, xma/layers/moe/__init__.py:54,79,104) go through the general
-        # pipeline, where they are added after each projection
-        if self.act is swiglu_packed and self.is_glu and self.c_fc.bias is None and self.c_proj.bias is None:
-            return _SwigluExperts.apply(
+        # biases: torch path only in the reference (xma/layers/moe/__init__.py:54,79,104); here both pipelines take them
+        activation = fused_activation_name(self.act, self.is_glu)
+        if activation is not None:
+            return _FusedExperts.apply(
                 hidden_states,
                 self.c_fc.weight,
                 self.c_proj.weight,
                 router_weights,
                 routing.sorted_scattered_idxs,
                 routing.expert_offsets,
+                self.c_fc.bias,
+                self.c_proj.bias,
+                activation,
             )
 
         hidden_states = self.c_fc.grouped_forward(

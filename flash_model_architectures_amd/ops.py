@@ -481,8 +481,9 @@ def _grouped_gemm(
     in_index: torch.Tensor | None = None,
     in_fan_out: int = 1,
     out_index: torch.Tensor | None = None,
+    bias: torch.Tensor | None = None,
 ) -> None:
-    nat.require_device(a, b, c, aux, expert_offsets, in_index, out_index)
+    nat.require_device(a, b, c, aux, expert_offsets, in_index, out_index, bias)
     _check_offsets(expert_offsets, E)
     if in_index is not None and out_index is not None:
         assert in_index.dtype == out_index.dtype
@@ -497,14 +498,28 @@ def _grouped_gemm(
     args.expert_offsets = expert_offsets.data_ptr()
     args.in_index, args.out_index = nat.ptr(in_index), nat.ptr(out_index)
     args.idx_is_i64, args.in_fan_out = _i64(index), in_fan_out
+    if bias is not None:
+        assert bias.dim() == 2 and bias.size(0) == E and bias.stride(1) == 1 and bias.dtype == a.dtype
+    args.bias, args.ld_bias = nat.ptr(bias), 0 if bias is None else _row_stride(bias)
     if kind != nat.GEMM_MT:
         ws_bytes = nat.load().xma_grouped_gemm_workspace_bytes(E, rows)
     else:
         ws_bytes = 16 * E  # the expert order of the weight-gradient kernel
     workspace = _workspace(a.device, ws_bytes)
     args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
-    tag = "xma_grouped_gemm/" + ("TN", "NN", "MT")[kind] + ("", "+swiglu", "+swiglu_bwd")[epilogue]
+    tag = "xma_grouped_gemm/" + ("TN", "NN", "MT")[kind] + _EPILOGUE_TAGS[epilogue]
     nat.call("xma_grouped_gemm", ctypes.byref(args), nat.stream(), tag=tag, flops=2.0 * rows * n * k)
+
+
+_EPILOGUE_TAGS = ("", "+swiglu", "+swiglu_bwd", "+glu", "+glu_bwd", "+gelu", "+gelu_bwd")
+
+# activation name -> (forward epilogue of the up-projection, backward epilogue of the down-projection's input
+# gradient, whether the pre-activation has two halves)
+FUSED_ACTIVATIONS = {
+    "swiglu": (nat.EPI_SWIGLU, nat.EPI_SWIGLU_BWD, True),
+    "glu": (nat.EPI_GLU, nat.EPI_GLU_BWD, True),
+    "gelu_tanh": (nat.EPI_GELU_TANH, nat.EPI_GELU_TANH_BWD, False),
+}
 
 
 def _weight_layout(W: torch.Tensor) -> tuple[int, int]:
@@ -529,15 +544,17 @@ def scatter2scatter(
     x_grouped: bool = False,
     y_grouped: bool = False,
     expert_offsets: torch.Tensor | None = None,
+    bias: torch.Tensor | None = None,
 ) -> None:
-    """out[o(p)] = X[i(p)] @ W[e(p)] over the grouped positions p.
+    """out[o(p)] = X[i(p)] @ W[e(p)] (+ bias[e(p)]) over the grouped positions p.
 
     i(p) = p if x_grouped else idx[p] // FAN_OUT; o(p) = p if y_grouped else idx[p]
     (xma/layers/moe/triton_implementation/scatter_kernel.py:105-108,128-131).  W is the logical
     [E, K, N] tensor; a permuted view of [E, N, K] storage is read in place.  The first eight parameters
     are the reference operator's (scatter_kernel.py:137-147); `expert_offsets` is an optional extra (either
     form, see `exclusive_offsets`) that saves the small kernel which otherwise recovers the offsets from
-    `sorted_expert_idxs`.
+    `sorted_expert_idxs`; `bias` [E, N] is another: it is added to the fp32 product inside the kernel when W is a
+    view of [E, N, K] storage (the forward projections), and by a separate pass otherwise.
     """
 
     assert sorted_scattered_idxs.size(0) == sorted_expert_idxs.size(0)
@@ -570,7 +587,10 @@ def scatter2scatter(
         in_index=None if x_grouped else idx,
         in_fan_out=FAN_OUT,
         out_index=None if y_grouped else idx,
+        bias=bias if kind == nat.GEMM_TN else None,
     )
+    if bias is not None and kind != nat.GEMM_TN:
+        add_expert_bias(y=out, bias=bias, sorted_expert_idxs=sorted_expert_idxs, out_index=None if y_grouped else idx)
 
 
 @xma_op(mutates_args={"DW"})
@@ -648,7 +668,7 @@ def group_bwd_W(
 
 
 @xma_op(mutates_args={"act", "preact"})
-def up_projection_swiglu(
+def up_projection_fused(
     X: torch.Tensor,
     W: torch.Tensor,
     sorted_scattered_idxs: torch.Tensor,
@@ -656,16 +676,22 @@ def up_projection_swiglu(
     act: torch.Tensor,
     preact: torch.Tensor | None,
     FAN_OUT: int,
+    activation: str,
+    bias: torch.Tensor | None = None,
 ) -> None:
-    """act[p] = swiglu_packed(X[idx[p] // FAN_OUT] @ W[e(p)]^T) with W stored [E, 2I, H] (up rows
-    first, gate rows second); `preact`, when given, receives the [M, 2I] product for backward."""
+    """act[p] = activation(X[idx[p] // FAN_OUT] @ W[e(p)]^T + bias[e(p)]) with W stored [E, N, H].
+
+    `activation` is a key of FUSED_ACTIVATIONS: "swiglu" (swiglu_packed: first half of the N rows is `up`, second
+    half `gate`, xma/functional/swiglu_packed.py:36), "glu" (torch.nn.GLU) or "gelu_tanh".  `preact`, when given,
+    receives the [M, N] pre-activation for backward."""
 
     E, N, K = W.shape
-    assert W.is_contiguous() and X.size(1) == K and act.size(1) * 2 == N
+    forward_epilogue, _, gated = FUSED_ACTIVATIONS[activation]
+    assert W.is_contiguous() and X.size(1) == K and act.size(1) * (2 if gated else 1) == N
     idx = sorted_scattered_idxs.contiguous()
     _grouped_gemm(
         kind=nat.GEMM_TN,
-        epilogue=nat.EPI_SWIGLU,
+        epilogue=forward_epilogue,
         E=E,
         rows=idx.size(0),
         n=N,
@@ -683,24 +709,28 @@ def up_projection_swiglu(
         ld_aux=0 if preact is None else _row_stride(preact),
         in_index=idx,
         in_fan_out=FAN_OUT,
+        bias=bias,
     )
 
 
 @xma_op(mutates_args={"d_preact"})
-def down_projection_dgrad_swiglu(
+def down_projection_dgrad_fused(
     DY: torch.Tensor,
     W: torch.Tensor,
     preact: torch.Tensor,
     expert_offsets: torch.Tensor,
     d_preact: torch.Tensor,
+    activation: str,
 ) -> None:
-    """d_preact = swiglu_packed'(preact) applied to (DY_grouped @ W[e]) with W stored [E, H, I]."""
+    """d_preact = activation'(preact) applied to (DY_grouped @ W[e]) with W stored [E, H, I]."""
 
     E, H, I = W.shape
-    assert W.is_contiguous() and DY.size(1) == H and preact.size(1) == 2 * I and d_preact.shape == preact.shape
+    _, backward_epilogue, gated = FUSED_ACTIVATIONS[activation]
+    assert W.is_contiguous() and DY.size(1) == H and preact.size(1) == (2 if gated else 1) * I
+    assert d_preact.shape == preact.shape
     _grouped_gemm(
         kind=nat.GEMM_NN,
-        epilogue=nat.EPI_SWIGLU_BWD,
+        epilogue=backward_epilogue,
         E=E,
         rows=DY.size(0),
         n=I,

@@ -37,7 +37,8 @@ enum xma_gemm_kind {
     XMA_GEMM_MT = 2
 };
 
-/* epilogues of xma_grouped_gemm */
+/* epilogues of xma_grouped_gemm: the activation between the two projections, fused into the up-projection
+   (TN kinds) and, for backward, into the input gradient of the down-projection (NN kinds) */
 enum xma_gemm_epilogue {
     XMA_EPI_NONE = 0,
     /* TN only.  B rows [0, N/2) are `up`, rows [N/2, N) are `gate` (xma/functional/swiglu_packed.py:36).
@@ -47,7 +48,20 @@ enum xma_gemm_epilogue {
     /* NN only.  The product is dAct[p, j], j < N.  `aux` holds the pre-activation [p, 0..2N)
        (up | gate).  Writes d_up into C[p, j] and d_gate into C[p, N + j] (ldc >= 2N), following
        xma/functional/swiglu/triton_implementation/backward.py:45-56. */
-    XMA_EPI_SWIGLU_BWD = 2
+    XMA_EPI_SWIGLU_BWD = 2,
+    /* TN only.  torch.nn.GLU over the last dimension, the activation of the reference's own MoE test
+       (tests/test_commons.py:93): act[p, j] = h[p, j] * sigmoid(h[p, N/2 + j]).  Operands as XMA_EPI_SWIGLU. */
+    XMA_EPI_GLU = 3,
+    /* NN only.  Backward of XMA_EPI_GLU, operands as XMA_EPI_SWIGLU_BWD: with a = h[p, j], b = h[p, N + j],
+       s = sigmoid(b): C[p, j] = d * s, C[p, N + j] = d * a * s * (1 - s). */
+    XMA_EPI_GLU_BWD = 4,
+    /* TN only.  tanh-approximated GELU (torch.nn.GELU(approximate="tanh"), tests/test_commons.py:94):
+       act[p, j] = 0.5 h (1 + tanh(sqrt(2/pi) (h + 0.044715 h^3))), j < N, into `C` (ldc >= N); the
+       pre-activation [p, 0..N) into `aux` when non-NULL (ld_aux >= N). */
+    XMA_EPI_GELU_TANH = 5,
+    /* NN only.  Backward of XMA_EPI_GELU_TANH: `aux` holds the pre-activation [p, 0..N); writes
+       C[p, j] = d * gelu'(h[p, j]), j < N (ldc >= N). */
+    XMA_EPI_GELU_TANH_BWD = 6
 };
 
 typedef struct xma_grouped_gemm_args {
@@ -80,6 +94,10 @@ typedef struct xma_grouped_gemm_args {
                                 16 * num_experts bytes; with it the 16-bit kernel walks the experts in descending
                                 order of their row counts, which balances the chip under skewed routing */
     int64_t workspace_bytes;
+    /* TN only, optional: per-expert bias [num_experts, N] (row stride ld_bias) added to the fp32 product before the
+       epilogue's activation and rounding: F.linear(x, W[e], bias[e]) of xma/layers/moe/__init__.py:103-106. */
+    const void* bias;
+    int64_t ld_bias;
 } xma_grouped_gemm_args;
 
 /* Description of the last failure on the calling thread ("" if none). */

@@ -1,4 +1,4 @@
-"""The ragged GEMM entry point in all three operand layouts and both fused epilogues, against
+"""The ragged GEMM entry point in all three operand layouts and with every fused epilogue, against
 per-expert fp32 matmuls on the CPU (the computation `Experts.torch_forward` performs,
 xma/layers/moe/__init__.py:103-106, and its transposes for the gradients)."""
 
@@ -63,11 +63,11 @@ def test_all_layouts_and_epilogues(case, dtype):
     # TN + SwiGLU epilogue
     act = torch.empty(M, I, dtype=dtype, device=dev)
     pre = torch.empty(M, 2 * I, dtype=dtype, device=dev)
-    ops.up_projection_swiglu(xd, w1d, idxd, offd, act, pre, k)
+    ops.up_projection_fused(xd, w1d, idxd, offd, act, pre, k, "swiglu")
     assert torch.equal(pre, h)  # same kernel body, same rounding
     assert_close(act, to.swiglu_packed(h.cpu()), tol, "fused swiglu")
     act2 = torch.empty_like(act)
-    ops.up_projection_swiglu(xd, w1d, idxd, offd, act2, None, k)  # inference: no pre-activation
+    ops.up_projection_fused(xd, w1d, idxd, offd, act2, None, k, "swiglu")  # inference: no pre-activation
     assert torch.equal(act2, act)
 
     # TN with row scatter: y_exp[idx[p]] = act[p] @ W2[e]^T
@@ -88,7 +88,7 @@ def test_all_layouts_and_epilogues(case, dtype):
 
     # NN + SwiGLU backward epilogue
     d_pre = torch.empty(M, 2 * I, dtype=dtype, device=dev)
-    ops.down_projection_dgrad_swiglu(dygd, w2d, pre, offd, d_pre)
+    ops.down_projection_dgrad_fused(dygd, w2d, pre, offd, d_pre, "swiglu")
     pc = pre.cpu()
     dg, du = to.swiglu_backward(pc[:, I:], pc[:, :I], d_act.cpu())
     assert_close(d_pre, torch.cat([du, dg], -1), tol, "fused swiglu backward")
@@ -118,6 +118,67 @@ def test_all_layouts_and_epilogues(case, dtype):
     d_w2_t = torch.empty(E, I, H, dtype=dtype, device=dev)
     ops.group_bwd_W(dygd, act, offd, d_w2_t, E)
     assert_close(d_w2_t, d_w2_ref.transpose(1, 2), tol, "down weight gradient, [E, K, N] storage")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("activation", ["swiglu", "glu", "gelu_tanh"])
+@pytest.mark.parametrize("case", [CASES[0], CASES[3], CASES[4]])
+def test_fused_activations_and_bias(case, activation, dtype):
+    """Every activation the epilogues fuse, forward and backward, with and without the per-expert bias that the
+    forward kernels add to the fp32 product: against the torch modules the reference's test drives the layer with
+    (tests/test_commons.py:93-94) evaluated in fp32 on the kernel's own (rounded) pre-activation, and against
+    autograd through them."""
+
+    T, H, I, E, k, empty = case
+    tol = TOL[dtype]
+    gated = activation != "gelu_tanh"
+    N = 2 * I if gated else I
+    module = {"swiglu": to.swiglu_packed, "glu": torch.nn.GLU(), "gelu_tanh": torch.nn.GELU(approximate="tanh")}[activation]
+    g = torch.Generator().manual_seed(T + H + I + E + len(activation))
+    x = torch.randn(T, H, generator=g).to(dtype)
+    w1 = (torch.randn(E, N, H, generator=g) * 0.05).to(dtype)
+    w2 = (torch.randn(E, H, I, generator=g) * 0.05).to(dtype)
+    b1 = (torch.randn(E, N, generator=g) * 0.5).to(dtype)
+    b2 = (torch.randn(E, H, generator=g) * 0.5).to(dtype)
+    r = _routing(T, E, k, T + E, empty)
+    idx, off = r.sorted_scattered_idxs, r.expert_offsets.tolist()
+    M, dev = T * k, "cuda"
+    idxd, offd, sed = idx.to(dev).int(), r.expert_offsets.to(dev), r.sorted_expert_idxs.to(dev).int()
+    xg = x[idx // k].float()
+    expert_of_row = r.sorted_expert_idxs
+
+    for bias in (None, b1):
+        act = torch.empty(M, I, dtype=dtype, device=dev)
+        pre = torch.full((M, N), float("nan"), dtype=dtype, device=dev)
+        ops.up_projection_fused(x.to(dev), w1.to(dev), idxd, offd, act, pre, k, activation,
+                                None if bias is None else bias.to(dev))
+        h_ref = _per_expert(off, lambda e, s: xg[s] @ w1[e].float().T)
+        if bias is not None:
+            h_ref = h_ref + bias.float()[expert_of_row]
+        assert_close(pre, h_ref, tol, f"pre-activation ({activation}, bias {bias is not None})")
+        assert_close(act, module(pre.float().cpu()), tol, f"fused {activation}")
+        without = torch.empty_like(act)
+        ops.up_projection_fused(x.to(dev), w1.to(dev), idxd, offd, without, None, k, activation,
+                                None if bias is None else bias.to(dev))
+        assert torch.equal(without, act)  # inference: no pre-activation kept, same values
+
+    # down projection with the bias inside the kernel, scattered rows
+    y_exp = torch.full((M, H), float("nan"), dtype=dtype, device=dev)
+    ops.scatter2scatter(act, w2.to(dev).permute(0, 2, 1), sed, idxd, y_exp, 1, True, False, offd, b2.to(dev))
+    a32 = act.float().cpu()
+    y_ref = torch.empty(M, H)
+    y_ref[idx] = _per_expert(off, lambda e, s: a32[s] @ w2[e].float().T) + b2.float()[expert_of_row]
+    assert_close(y_exp, y_ref, tol, "down projection with bias")
+
+    # backward epilogue: d_pre = activation'(pre) * (dY_grouped @ W2[e]) against autograd through the module
+    dyg = torch.randn(M, H, generator=g).to(dtype)
+    d_pre = torch.full((M, N), float("nan"), dtype=dtype, device=dev)
+    ops.down_projection_dgrad_fused(dyg.to(dev), w2.to(dev), pre, offd, d_pre, activation)
+    d_act = torch.empty(M, I, dtype=dtype, device=dev)
+    ops.scatter2scatter(dyg.to(dev), w2.to(dev), sed, idxd, d_act, 1, True, True, offd)
+    leaf = pre.float().cpu().requires_grad_()
+    module(leaf).backward(d_act.float().cpu())
+    assert_close(d_pre, leaf.grad, tol, f"fused {activation} backward")
 
 
 def test_argument_validation():
