@@ -831,49 +831,61 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                 pin(ups[it2]);
                 pin(gates[it2]);
             }
+            // one copy of the loop per activation, chosen once: inside it the activation is a constant
+            auto rows = [&](auto act_tag) {
+                constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
-            for (int it2 = 0; it2 < IT / 2; ++it2) {
-                const int32_t row_out = odd ? out_row[2 * it2 + 1] : out_row[2 * it2];
-                const int br = etid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
-                if (row_out < 0 || j >= half_n) continue;
-                const int64_t p = m_begin + tile_row(mi, br);
-                const u32x4_t up = ups[it2], gate = gates[it2];
-                if (P.aux) {
-                    T* h = reinterpret_cast<T*>(P.aux) + p * P.ld_aux;
-                    *reinterpret_cast<u32x4_t*>(h + j) = up;
-                    *reinterpret_cast<u32x4_t*>(h + half_n + j) = gate;
+                for (int it2 = 0; it2 < IT / 2; ++it2) {
+                    const int32_t row_out = odd ? out_row[2 * it2 + 1] : out_row[2 * it2];
+                    const int br = etid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
+                    if (row_out < 0 || j >= half_n) continue;
+                    const int64_t p = m_begin + tile_row(mi, br);
+                    const u32x4_t up = ups[it2], gate = gates[it2];
+                    if (P.aux) {
+                        T* h = reinterpret_cast<T*>(P.aux) + p * P.ld_aux;
+                        *reinterpret_cast<u32x4_t*>(h + j) = up;
+                        *reinterpret_cast<u32x4_t*>(h + half_n + j) = gate;
+                    }
+                    float u[PV], g[PV], o[PV];
+                    Elem<T>::unpack(to_uint4(up), u);
+                    Elem<T>::unpack(to_uint4(gate), g);
+#pragma unroll
+                    for (int q = 0; q < PV; ++q) o[q] = gated_forward<true>(ACT, u[q], g[q]);
+                    *reinterpret_cast<uint4*>(C + (int64_t)row_out * P.ldc + j) = Elem<T>::pack(o);
                 }
-                float u[PV], g[PV], o[PV];
-                Elem<T>::unpack(to_uint4(up), u);
-                Elem<T>::unpack(to_uint4(gate), g);
-#pragma unroll
-                for (int q = 0; q < PV; ++q) o[q] = gated_forward<true>(P.act, u[q], g[q]);
-                *reinterpret_cast<uint4*>(C + (int64_t)row_out * P.ldc + j) = Elem<T>::pack(o);
-            }
-        } else {  // XMA_EPI_SWIGLU_BWD
+            };
+            if (P.act == ACT_SWIGLU) rows(std::integral_constant<int, ACT_SWIGLU>{});
+            else rows(std::integral_constant<int, ACT_GLU>{});
+        } else {  // EPI_BACKWARD
             const int64_t n = n0 + cc * PV;
             if constexpr (mi + 1 < MI) load_saved(mi + 1, hu[(mi + 1) & 1], hg[(mi + 1) & 1]);
             u32x4_t dv[IT];
             read_own_chunks(dv);
+            auto rows = [&](auto act_tag) {
+                constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
-            for (int it = 0; it < IT; ++it) {
-                if (out_row[it] < 0 || n >= P.n) continue;
-                float u[PV], g[PV], d[PV], du[PV], dg[PV];
-                Elem<T>::unpack(to_uint4(hu[mi & 1][it]), u);
-                Elem<T>::unpack(to_uint4(hg[mi & 1][it]), g);
-                Elem<T>::unpack(to_uint4(dv[it]), d);
-                T* out = C + (int64_t)out_row[it] * P.ldc;
-                if (P.act == ACT_GELU_TANH) {
+                for (int it = 0; it < IT; ++it) {
+                    if (out_row[it] < 0 || n >= P.n) continue;
+                    float u[PV], g[PV], d[PV], du[PV], dg[PV];
+                    Elem<T>::unpack(to_uint4(hu[mi & 1][it]), u);
+                    Elem<T>::unpack(to_uint4(hg[mi & 1][it]), g);
+                    Elem<T>::unpack(to_uint4(dv[it]), d);
+                    T* out = C + (int64_t)out_row[it] * P.ldc;
+                    if constexpr (ACT == ACT_GELU_TANH) {
 #pragma unroll
-                    for (int q = 0; q < PV; ++q) du[q] = gelu_tanh_backward<true>(u[q], d[q]);
-                    *reinterpret_cast<uint4*>(out + n) = Elem<T>::pack(du);
-                } else {
+                        for (int q = 0; q < PV; ++q) du[q] = gelu_tanh_backward<true>(u[q], d[q]);
+                        *reinterpret_cast<uint4*>(out + n) = Elem<T>::pack(du);
+                    } else {
 #pragma unroll
-                    for (int q = 0; q < PV; ++q) gated_backward<true>(P.act, u[q], g[q], d[q], du[q], dg[q]);
-                    *reinterpret_cast<uint4*>(out + n) = Elem<T>::pack(du);
-                    *reinterpret_cast<uint4*>(out + P.n + n) = Elem<T>::pack(dg);
+                        for (int q = 0; q < PV; ++q) gated_backward<true>(ACT, u[q], g[q], d[q], du[q], dg[q]);
+                        *reinterpret_cast<uint4*>(out + n) = Elem<T>::pack(du);
+                        *reinterpret_cast<uint4*>(out + P.n + n) = Elem<T>::pack(dg);
+                    }
                 }
-            }
+            };
+            if (P.act == ACT_SWIGLU) rows(std::integral_constant<int, ACT_SWIGLU>{});
+            else if (P.act == ACT_GLU) rows(std::integral_constant<int, ACT_GLU>{});
+            else rows(std::integral_constant<int, ACT_GELU_TANH>{});
         }
     };
     store_rows(slab<0>(), std::integral_constant<int, 0>{}, orow[0]);
