@@ -87,9 +87,75 @@ __global__ __launch_bounds__(256) void count_kernel(const IdT* __restrict__ ids,
     }
 }
 
+// Small inputs: ONE block builds the whole histogram in LDS (one replica per wave, summed at the end) and writes
+// every bin, so the output needs no clearing beforehand and the call is a single launch.
+constexpr int64_t kSingleBlockIds = (int64_t)1 << 15;  // most ids a single block is given (two chunks per wave)
+constexpr int kSingleBlockBins = 512;                  // most bins (16 replicas of 2 KiB in LDS)
+template <typename IdT>
+__global__ __launch_bounds__(1024) void count_single_block_kernel(const IdT* __restrict__ ids, int64_t n, int bins,
+                                                                   uint32_t* __restrict__ counts) {
+    extern __shared__ uint32_t lds_hist[];
+    constexpr int kWaves = 1024 / kWaveSize;
+    for (int i = threadIdx.x; i < bins * kWaves; i += 1024) lds_hist[i] = 0;
+    __syncthreads();
+    uint32_t* mine = lds_hist + (threadIdx.x / kWaveSize) * bins;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) {
+        const IdT e = ids[i];
+        if (e >= 0 && e < bins) atomicAdd(&mine[e], 1u);
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < bins; b += 1024) {
+        uint32_t c = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) c += lds_hist[w * bins + b];
+        counts[b] = c;
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // stable counting sort
 // ------------------------------------------------------------------------------------------
+// A wave reads its ids kChunk at a time: 16 per lane, requested together (the walk over a chunk is otherwise a chain
+// of dependent load latencies), -1 past `end`.
+constexpr int kBatches = kChunk / kWaveSize;
+template <typename IdT>
+__device__ __forceinline__ void load_chunk(const IdT* __restrict__ ids, int64_t begin, int64_t end, int lane,
+                                           int64_t (&v)[kBatches]) {
+#pragma unroll
+    for (int j = 0; j < kBatches; ++j) {
+        const int64_t i = begin + j * kWaveSize + lane;
+        v[j] = i < end ? (int64_t)ids[i] : -1;
+    }
+}
+
+// One 64-wide batch of the placement: lanes holding the same expert id find each other with log2(E) ballots, the
+// first of them takes popcount(peers) consecutive slots from next[e], and every lane's slot follows from its rank
+// among its peers, so equal ids keep their order.
+template <typename OutT>
+__device__ __forceinline__ void place_batch(int64_t e64, int64_t i, int E, int nbits, int lane, uint32_t* next,
+                                            OutT* __restrict__ sorted_ids, OutT* __restrict__ perm) {
+    const bool ok = e64 >= 0 && e64 < E;
+    const uint32_t e = ok ? (uint32_t)e64 : 0u;
+    uint64_t peers = __ballot(ok);
+    for (int b = 0; b < nbits; ++b) {
+        const bool bit = (e >> b) & 1u;
+        const uint64_t bal = __ballot(ok && bit);
+        peers &= bit ? bal : ~bal;
+    }
+    uint32_t base = 0;
+    const int leader = ok ? (int)__ffsll((unsigned long long)peers) - 1 : lane;
+    if (ok && leader == lane) {
+        base = next[e];
+        next[e] = base + (uint32_t)__popcll(peers);
+    }
+    base = __shfl(base, leader, kWaveSize);
+    if (ok) {
+        const uint32_t pos = base + (uint32_t)__popcll(peers & (((uint64_t)1 << lane) - 1));
+        perm[pos] = (OutT)i;
+        sorted_ids[pos] = (OutT)e;
+    }
+}
+
 template <typename IdT>
 __global__ __launch_bounds__(256) void unit_hist_kernel(const IdT* __restrict__ ids, int64_t n, int E,
                                                          int waves_per_block, uint32_t* __restrict__ unit_hist) {
@@ -103,10 +169,11 @@ __global__ __launch_bounds__(256) void unit_hist_kernel(const IdT* __restrict__ 
     const int64_t begin = unit * kChunk;
     if (begin < n) {
         const int64_t end = begin + kChunk < n ? begin + kChunk : n;
-        for (int64_t i = begin + lane; i < end; i += kWaveSize) {
-            IdT e = ids[i];
-            if (e >= 0 && e < E) atomicAdd(&mine[e], 1u);
-        }
+        int64_t v[kBatches];
+        load_chunk(ids, begin, end, lane, v);
+#pragma unroll
+        for (int j = 0; j < kBatches; ++j)
+            if (v[j] >= 0 && v[j] < E) atomicAdd(&mine[v[j]], 1u);
     }
     __syncthreads();
     if (begin < n) {
@@ -230,32 +297,91 @@ __global__ __launch_bounds__(256) void place_kernel(const IdT* __restrict__ ids,
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
 
     const int64_t end = begin + kChunk < n ? begin + kChunk : n;
-    const uint64_t lt_mask = ((uint64_t)1 << lane) - 1;
-    for (int64_t i0 = begin; i0 < end; i0 += kWaveSize) {
-        const int64_t i = i0 + lane;
-        const bool live = i < end;
-        int64_t e64 = live ? (int64_t)ids[i] : -1;
-        const bool ok = live && e64 >= 0 && e64 < E;
-        const uint32_t e = ok ? (uint32_t)e64 : 0u;
-        // lanes holding the same expert id as this lane
-        uint64_t peers = __ballot(ok);
-        for (int b = 0; b < nbits; ++b) {
-            const bool bit = (e >> b) & 1u;
-            const uint64_t bal = __ballot(ok && bit);
-            peers &= bit ? bal : ~bal;
+    int64_t v[kBatches];
+    load_chunk(ids, begin, end, lane, v);
+#pragma unroll
+    for (int j = 0; j < kBatches; ++j)
+        place_batch(v[j], begin + j * kWaveSize + lane, E, nbits, lane, next, sorted_ids, perm);
+}
+
+// The whole counting sort in ONE block of 16 waves, for up to kSingleBlockIds ids and kSingleBlockBins experts (the
+// routed rows of one MoE layer): wave w owns the w-th contiguous run of ids.  (1) every wave builds the histogram
+// of its run in its own LDS row; (2) thread e turns column e into exclusive prefixes over the waves, the block
+// scans the column totals into the expert offsets, and the two are added up: row w, column e is then the first
+// output slot of wave w's ids of expert e; (3) every wave walks its run again in order and ranks equal ids inside
+// each 64-wide batch with ballots, as place_kernel does.  No workspace, no other launch.
+template <typename IdT, typename OutT>
+__global__ __launch_bounds__(1024) void route_single_block_kernel(const IdT* __restrict__ ids, int64_t n, int E,
+                                                                   int nbits, uint32_t* __restrict__ counts,
+                                                                   int32_t* __restrict__ offsets,
+                                                                   OutT* __restrict__ sorted_ids,
+                                                                   OutT* __restrict__ perm) {
+    extern __shared__ uint32_t lds_hist[];  // [16 waves][E], then [1024] for the scan
+    constexpr int kWaves = 1024 / kWaveSize;
+    uint32_t* part = lds_hist + kWaves * E;
+    const int wave = threadIdx.x / kWaveSize;
+    const int lane = lane_id();
+    for (int i = threadIdx.x; i < kWaves * E; i += 1024) lds_hist[i] = 0;
+    __syncthreads();
+
+    const int64_t per = ((n + kWaves - 1) / kWaves + kWaveSize - 1) / kWaveSize * kWaveSize;  // ids per wave
+    const int64_t begin = wave * per < n ? wave * per : n;
+    const int64_t end = begin + per < n ? begin + per : n;
+    uint32_t* mine = lds_hist + wave * E;
+    int64_t v[kBatches];  // the wave's first chunk stays in registers for the placement
+    load_chunk(ids, begin, end, lane, v);
+#pragma unroll
+    for (int j = 0; j < kBatches; ++j)
+        if (v[j] >= 0 && v[j] < E) atomicAdd(&mine[v[j]], 1u);
+    for (int64_t c0 = begin + kChunk; c0 < end; c0 += kChunk) {
+        int64_t u[kBatches];
+        load_chunk(ids, c0, end, lane, u);
+#pragma unroll
+        for (int j = 0; j < kBatches; ++j)
+            if (u[j] >= 0 && u[j] < E) atomicAdd(&mine[u[j]], 1u);
+    }
+    __syncthreads();
+
+    // column e: exclusive prefixes over the waves, total -> counts
+    const int e_mine = threadIdx.x;
+    uint32_t total = 0;
+    if (e_mine < E) {
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const uint32_t c = lds_hist[w * E + e_mine];
+            lds_hist[w * E + e_mine] = total;
+            total += c;
         }
-        uint32_t base = 0;
-        const int leader = ok ? (int)__ffsll((unsigned long long)peers) - 1 : lane;
-        if (ok && leader == lane) {
-            base = next[e];
-            next[e] = base + (uint32_t)__popcll(peers);
-        }
-        base = __shfl(base, leader, kWaveSize);
-        if (ok) {
-            const uint32_t pos = base + (uint32_t)__popcll(peers & lt_mask);
-            perm[pos] = (OutT)i;
-            sorted_ids[pos] = (OutT)e;
-        }
+        counts[e_mine] = total;
+    }
+    // exclusive scan of the totals over the experts (Hillis-Steele over 1024 slots)
+    part[threadIdx.x] = total;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        const uint32_t v = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+        __syncthreads();
+        part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    const uint32_t first_slot = part[threadIdx.x] - total;
+    if (e_mine < E) {
+        offsets[e_mine] = (int32_t)first_slot;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) lds_hist[w * E + e_mine] += first_slot;
+    }
+    if (threadIdx.x == 1023) offsets[E] = (int32_t)part[1023];
+    __syncthreads();
+
+    // placement, stable inside the wave's run and across the runs
+    uint32_t* next = mine;
+#pragma unroll
+    for (int j = 0; j < kBatches; ++j)
+        place_batch(v[j], begin + j * kWaveSize + lane, E, nbits, lane, next, sorted_ids, perm);
+    for (int64_t c0 = begin + kChunk; c0 < end; c0 += kChunk) {
+        load_chunk(ids, c0, end, lane, v);
+#pragma unroll
+        for (int j = 0; j < kBatches; ++j)
+            place_batch(v[j], c0 + j * kWaveSize + lane, E, nbits, lane, next, sorted_ids, perm);
     }
 }
 
@@ -451,6 +577,16 @@ int xma_continuous_count(const void* ids, int ids_is_i64, int64_t n, int32_t bin
     XMA_REQUIRE(bins >= 1 && bins <= kMaxExperts, "xma_continuous_count: bins=%d outside [1, %d]", bins, kMaxExperts);
     XMA_REQUIRE(n >= 0 && n < ((int64_t)1 << 32), "xma_continuous_count: n=%lld does not fit uint32", (long long)n);
     XMA_REQUIRE(counts != nullptr && (ids != nullptr || n == 0), "xma_continuous_count: null pointer");
+    if (n <= kSingleBlockIds && bins <= kSingleBlockBins) {  // one launch, writes every bin
+        const size_t lds = (size_t)bins * (1024 / kWaveSize) * sizeof(uint32_t);
+        if (ids_is_i64)
+            hipLaunchKernelGGL(count_single_block_kernel<int64_t>, dim3(1), dim3(1024), lds, stream, (const int64_t*)ids, n,
+                               (int)bins, counts);
+        else
+            hipLaunchKernelGGL(count_single_block_kernel<int32_t>, dim3(1), dim3(1024), lds, stream, (const int32_t*)ids, n,
+                               (int)bins, counts);
+        return check_launch("xma_continuous_count");
+    }
     hipLaunchKernelGGL(fill_u32_kernel, dim3((bins + 255) / 256), dim3(256), 0, stream, counts, (int64_t)bins, 0u);
     if (n > 0) {
         int copies = 2048 / bins;
@@ -488,6 +624,26 @@ static int route_build_launch(const void* ids, int ids_is_i64, int64_t n, int32_
                            (int64_t)E + 1, 0u);
         return check_launch("xma_route_build");
     }
+    const int nbits = ceil_log2(E);
+    if (n <= kSingleBlockIds && E <= kSingleBlockBins) {  // one launch, no workspace
+        const size_t lds_one = ((size_t)E * (1024 / kWaveSize) + 1024) * sizeof(uint32_t);
+#define XMA_ROUTE_ONE(IdT, OutT)                                                                                     \
+    hipLaunchKernelGGL((route_single_block_kernel<IdT, OutT>), dim3(1), dim3(1024), lds_one, stream, (const IdT*)ids, \
+                       n, (int)E, nbits, counts, offsets, (OutT*)sorted_ids, (OutT*)perm)
+        if (ids_is_i64) {
+            if (out_is_i64)
+                XMA_ROUTE_ONE(int64_t, int64_t);
+            else
+                XMA_ROUTE_ONE(int64_t, int32_t);
+        } else {
+            if (out_is_i64)
+                XMA_ROUTE_ONE(int32_t, int64_t);
+            else
+                XMA_ROUTE_ONE(int32_t, int32_t);
+        }
+#undef XMA_ROUTE_ONE
+        return check_launch("xma_route_build");
+    }
     const int64_t units = ceil_div(n, kChunk);
     const int wpb = sort_waves_per_block(E);
     const unsigned blocks = (unsigned)ceil_div(units, wpb);
@@ -502,7 +658,6 @@ static int route_build_launch(const void* ids, int ids_is_i64, int64_t n, int32_
     hipLaunchKernelGGL(unit_scan_kernel, dim3((E + kWaveSize - 1) / kWaveSize), dim3(1024), 0, stream, unit_hist, units,
                        (int)E, counts);
     hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, stream, (const uint32_t*)counts, (int)E, offsets);
-    const int nbits = ceil_log2(E);
 #define XMA_PLACE(IdT, OutT)                                                                                       \
     hipLaunchKernelGGL((place_kernel<IdT, OutT>), dim3(blocks), dim3(wpb * kWaveSize), lds, stream, (const IdT*)ids, \
                        n, (int)E, nbits, wpb, (const uint32_t*)unit_hist, (const int32_t*)offsets,                 \
