@@ -66,6 +66,7 @@ inline void split_epilogue(int epilogue, int& shape, int& act) {
 constexpr int kSplitSlots = 256;
 constexpr int kMaxSplit = 4;
 constexpr int kSplitMaxRounds = 8;
+constexpr int kSplitMinStages = 32;  // a part must keep this many 64-deep stages of the reduction
 constexpr int64_t kSplitTileFloats = 256 * 256;
 inline int64_t tile_table_bytes(int64_t row_tiles) { return ((4 + 2 * row_tiles) * (int64_t)sizeof(int32_t) + 255) / 256 * 256; }
 inline int64_t split_region_bytes() {
@@ -193,10 +194,14 @@ __device__ __forceinline__ bool locate_tile(int row_tiles, int col_tiles, int& r
 
 // Row-grouped kinds with split-K of the remainder.  With T tiles on a device of C compute units the first
 // floor(T / C) * C tiles fill whole rounds; the R = T mod C tiles of the last round would leave C - R units idle
-// for a whole tile time, so each of them is cut along the reduction into S = min(kMaxSplit, C / R, stages)
-// parts that run side by side.  (Only when the launch has fewer than kSplitMaxRounds rounds: the idle units of
-// a last round matter less the more rounds there are, and the parts cost a reduction.)  Work-groups are dealt per XCD as in locate_tile<false>: XCD x takes the x-th
-// eighth of the whole tiles, then the x-th eighth of the parts (part-major, so neighbours share panels).
+// for a whole tile time, so each of them is cut along the reduction into S = min(kMaxSplit, C / R,
+// stages / kSplitMinStages) parts that run side by side.  Only when the launch has fewer than kSplitMaxRounds
+// rounds (the idle units of a last round matter less the more rounds there are), and only while a part keeps
+// kSplitMinStages stages: every part parks a 256 KiB tile of fp32 sums in HBM and the last one reads them all
+// back, which costs about as much as 16 stages of the main loop (measured: reductions of 2048 split in two lose
+// 20 % of the launch, reductions of 14336 split in three gain 8 %).  Work-groups are dealt per XCD as in
+// locate_tile<false>: XCD x takes the x-th eighth of the whole tiles, then the x-th eighth of the parts
+// (part-major, so neighbours share panels).
 struct TileWork {
     int row_tile, col_tile;
     int part, parts;  // this work-group reduces stages [part * n / parts, (part + 1) * n / parts)
@@ -211,7 +216,7 @@ __device__ __forceinline__ bool locate_work(int row_tiles, int col_tiles, int nu
     const int rem = total - whole;
     int parts = rem > 0 && total < kSplitMaxRounds * num_cu ? num_cu / rem : 1;
     parts = parts > kMaxSplit ? kMaxSplit : parts;
-    parts = parts > stages ? (int)stages : parts;
+    parts = parts > stages / kSplitMinStages ? (int)(stages / kSplitMinStages) : parts;
     parts = parts < 1 ? 1 : parts;
     const int whole_per_xcd = whole / kNumXcd;
     int tile;

@@ -807,7 +807,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 #pragma unroll
                 for (int it = 0; it < IT; ++it)
                     if (out_row[it] >= 0 && n < P.n)
-                        *reinterpret_cast<u32x4_t*>(C + (int64_t)out_row[it] * P.ldc + n) = v[it];
+                        __builtin_nontemporal_store(v[it], reinterpret_cast<u32x4_t*>(C + (int64_t)out_row[it] * P.ldc + n));
             }
         } else if constexpr (EPI == EPI_PAIRED) {
             // The slab row holds 16 chunks of the up half, then the 16 matching chunks of the gate half.  Thread
@@ -843,15 +843,15 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                     const u32x4_t up = ups[it2], gate = gates[it2];
                     if (P.aux) {
                         T* h = reinterpret_cast<T*>(P.aux) + p * P.ld_aux;
-                        *reinterpret_cast<u32x4_t*>(h + j) = up;
-                        *reinterpret_cast<u32x4_t*>(h + half_n + j) = gate;
+                        __builtin_nontemporal_store(up, reinterpret_cast<u32x4_t*>(h + j));
+                        __builtin_nontemporal_store(gate, reinterpret_cast<u32x4_t*>(h + half_n + j));
                     }
                     float u[PV], g[PV], o[PV];
                     Elem<T>::unpack(to_uint4(up), u);
                     Elem<T>::unpack(to_uint4(gate), g);
 #pragma unroll
                     for (int q = 0; q < PV; ++q) o[q] = gated_forward<true>(ACT, u[q], g[q]);
-                    *reinterpret_cast<uint4*>(C + (int64_t)row_out * P.ldc + j) = Elem<T>::pack(o);
+                    { const uint4 pk = Elem<T>::pack(o); __builtin_nontemporal_store(u32x4_t{pk.x, pk.y, pk.z, pk.w}, reinterpret_cast<u32x4_t*>(C + (int64_t)row_out * P.ldc + j)); }
                 }
             };
             if (P.act == ACT_SWIGLU) rows(std::integral_constant<int, ACT_SWIGLU>{});
@@ -878,8 +878,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                     } else {
 #pragma unroll
                         for (int q = 0; q < PV; ++q) gated_backward<true>(ACT, u[q], g[q], d[q], du[q], dg[q]);
-                        *reinterpret_cast<uint4*>(out + n) = Elem<T>::pack(du);
-                        *reinterpret_cast<uint4*>(out + P.n + n) = Elem<T>::pack(dg);
+                        { const uint4 a = Elem<T>::pack(du), b = Elem<T>::pack(dg); __builtin_nontemporal_store(u32x4_t{a.x, a.y, a.z, a.w}, reinterpret_cast<u32x4_t*>(out + n)); __builtin_nontemporal_store(u32x4_t{b.x, b.y, b.z, b.w}, reinterpret_cast<u32x4_t*>(out + P.n + n)); }
                     }
                 }
             };

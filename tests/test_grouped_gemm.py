@@ -222,11 +222,12 @@ def test_ragged_tail_rows_are_not_touched():
 @pytest.mark.parametrize("layout", ["TN", "NN"])
 def test_whole_rounds_plus_split_remainder(layout):
     """More tiles than compute units, with a remainder: the first tiles run whole, the tiles of the last,
-    partly filled round are reduced in parts and summed by the part that finishes last.  Checked against fp32
+    partly filled round are reduced in parts and summed by the part that finishes last (a part keeps at least 32
+    stages of 64, so the reduction must be long: 6200 = 96 stages and a tail, cut in three).  Checked against fp32
     matmuls on the device; run twice to see that the result does not depend on the arrival order."""
 
     dev = "cuda"
-    E, K, N = 4, 320, 1792  # 7 column tiles; ~43 row tiles -> ~300 tiles on 256 compute units
+    E, K, N = 4, 6200, 1792  # 7 column tiles; ~43 row tiles -> ~300 tiles on 256 compute units
     sizes = [2700, 1, 3100, 4300]
     M = sum(sizes)
     g = torch.Generator().manual_seed(3)
