@@ -642,41 +642,48 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     // Per-lane coordinates are derived from a fresh, opaque copy of the thread index: derived from `tid` they
     // would be the values computed before the main loop, which the compiler then keeps in scratch memory
     // across the loop and reloads in the middle of the epilogue's batched requests.
+    // A wave that is alone on its SIMD issues one vector instruction every 4-5 cycles, so this part of the kernel
+    // is bound by its instruction count: row arithmetic is 32-bit and relative to the tile (the thread's first
+    // buffer row r0 plus a compile-time constant), and whether a row exists is one compare against a scalar where
+    // the row is used, not a mark kept per row.
     const int etid = opaque(tid);
-    const int cc = etid % C_CHUNKS;
-    auto buffer_row = [&](int it) { return etid / C_CHUNKS + it * ROW_STEP; };
-    auto tile_row = [&](int mi, int br) { return (br >> 5) * 128 + mi * 32 + (br & 31); };
+    const int cc = etid & (C_CHUNKS - 1);
+    const int r0 = (etid / C_CHUNKS) & (ROW_STEP - 1);
+    auto buffer_row = [&](int it) { return r0 + it * ROW_STEP; };
+    // tile row of buffer row r0 + 8 * it of slab mi, less r0: buffer rows 0..31 are tile rows mi*32 + 0..31, buffer
+    // rows 32..63 the same rows of the lower wave row (+128)
+    auto row_base = [](int mi, int it) { return (it >> 2) * 128 + mi * 32 + (it & 3) * ROW_STEP; };
+    const int rows_here = (int)(m_end - m_begin);  // 1..256
+    auto row_exists = [&](int mi, int it) { return r0 < rows_here - row_base(mi, it); };
+    // a row of the tile that exists: the wanted one or, past the end, the last one
+    auto safe_row = [&](int mi, int it) {
+        const int r = r0 + row_base(mi, it);
+        return (uint32_t)(r < rows_here ? r : rows_here - 1);
+    };
 
-    int32_t orow[MI][IT];  // output row of each owned row, -1: past the end of the expert's rows
-    // Branch-free: rows past the end read the index of the expert's last row and are marked afterwards.  (Putting
-    // off the marking until the accumulators have gone to LDS, to overlap the index loads with that copy,
-    // measured no gain.)
+    int32_t orow[MI][IT];  // output row of each owned row (of the last existing row for rows past the end)
     if constexpr (KIND != XMA_GEMM_MT) {
-        const int64_t last = m_end - 1;
         auto fill = [&](auto index_of) {
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-                for (int it = 0; it < IT; ++it) {
-                    const int64_t p = m_begin + tile_row(mi, buffer_row(it));
-                    orow[mi][it] = index_of(p < m_end ? p : last);
-                }
+                for (int it = 0; it < IT; ++it) orow[mi][it] = index_of(safe_row(mi, it));
             batch_fence();
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-                for (int it = 0; it < IT; ++it) {
-                    const int64_t p = m_begin + tile_row(mi, buffer_row(it));
-                    pin(orow[mi][it]);
-                    orow[mi][it] = p < m_end ? orow[mi][it] : -1;
-                }
+                for (int it = 0; it < IT; ++it) pin(orow[mi][it]);
         };
-        if (EPI == EPI_BACKWARD || P.out_index == nullptr)  // that epilogue only writes grouped rows
-            fill([&](int64_t p) { return (int32_t)p; });
-        else if (P.idx_is_i64)
-            fill([&](int64_t p) { return (int32_t)reinterpret_cast<const int64_t*>(P.out_index)[p]; });
-        else
-            fill([&](int64_t p) { return reinterpret_cast<const int32_t*>(P.out_index)[p]; });
+        if (EPI == EPI_BACKWARD || P.out_index == nullptr) {  // that epilogue only writes grouped rows
+            const int32_t first = (int32_t)m_begin;
+            fill([&](uint32_t r) { return first + (int32_t)r; });
+        } else if (P.idx_is_i64) {
+            const int64_t* index = reinterpret_cast<const int64_t*>(P.out_index) + m_begin;
+            fill([&](uint32_t r) { return (int32_t)index[r]; });
+        } else {
+            const int32_t* index = reinterpret_cast<const int32_t*>(P.out_index) + m_begin;
+            fill([&](uint32_t r) { return index[r]; });
+        }
     }
 
     // Activation backward: the saved pre-activation chunks (the two halves of a gated one; tanh-GELU has a single
@@ -690,8 +697,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         const int64_t second_half = P.act == ACT_GELU_TANH ? 0 : P.n;
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
-            const int64_t p = m_begin + tile_row(mi, buffer_row(it));
-            const T* h = reinterpret_cast<const T*>(P.aux) + (p < m_end ? p : m_end - 1) * P.ld_aux;
+            const T* h = reinterpret_cast<const T*>(P.aux) + (m_begin + safe_row(mi, it)) * P.ld_aux;
             up[it] = *reinterpret_cast<const u32x4_t*>(h + n);
             gate[it] = *reinterpret_cast<const u32x4_t*>(h + second_half + n);
         }
@@ -781,7 +787,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             read_own_chunks(v);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                const int64_t i = tile_i0 + tile_row(mi, buffer_row(it));
+                const int64_t i = tile_i0 + r0 + row_base(mi, it);
                 // streaming store: a weight gradient is read again only by the optimizer, so it should not push the
                 // operand panels of the running tiles out of the caches (1-2 % on this kind)
                 if (i < P.n && j < P.k) __builtin_nontemporal_store(v[it], reinterpret_cast<u32x4_t*>(out + i * P.ldc));
@@ -794,8 +800,8 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                 // tanh-GELU of the product; the rounded product itself is kept as the pre-activation
 #pragma unroll
                 for (int it = 0; it < IT; ++it) {
-                    if (out_row[it] < 0 || n >= P.n) continue;
-                    const int64_t p = m_begin + tile_row(mi, buffer_row(it));
+                    if (!row_exists(mi, it) || n >= P.n) continue;
+                    const int64_t p = m_begin + r0 + row_base(mi, it);
                     if (P.aux) *reinterpret_cast<u32x4_t*>(reinterpret_cast<T*>(P.aux) + p * P.ld_aux + n) = v[it];
                     float h[PV], o[PV];
                     Elem<T>::unpack(to_uint4(v[it]), h);
@@ -806,7 +812,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             } else {
 #pragma unroll
                 for (int it = 0; it < IT; ++it)
-                    if (out_row[it] >= 0 && n < P.n)
+                    if (row_exists(mi, it) && n < P.n)
                         __builtin_nontemporal_store(v[it], reinterpret_cast<u32x4_t*>(C + (int64_t)out_row[it] * P.ldc + n));
             }
         } else if constexpr (EPI == EPI_PAIRED) {
@@ -818,10 +824,11 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             const int pair = cc % HALF_CHUNKS;
             const int64_t j = n0 + pair * PV;
             const bool odd = cc >= HALF_CHUNKS;
+            const int r1 = r0 + (odd ? ROW_STEP : 0);  // the thread's first buffer row among those it computes
             u32x4_t ups[IT / 2], gates[IT / 2];
 #pragma unroll
             for (int it2 = 0; it2 < IT / 2; ++it2) {
-                const int br = etid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
+                const int br = r1 + 2 * it2 * ROW_STEP;
                 ups[it2] = chunk_at(br, pair);
                 gates[it2] = chunk_at(br, pair + HALF_CHUNKS);
             }
@@ -837,9 +844,8 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 #pragma unroll
                 for (int it2 = 0; it2 < IT / 2; ++it2) {
                     const int32_t row_out = odd ? out_row[2 * it2 + 1] : out_row[2 * it2];
-                    const int br = etid / C_CHUNKS + (2 * it2 + (odd ? 1 : 0)) * ROW_STEP;
-                    if (row_out < 0 || j >= half_n) continue;
-                    const int64_t p = m_begin + tile_row(mi, br);
+                    if (r1 >= rows_here - row_base(mi, 2 * it2) || j >= half_n) continue;
+                    const int64_t p = m_begin + r1 + row_base(mi, 2 * it2);
                     const u32x4_t up = ups[it2], gate = gates[it2];
                     if (P.aux) {
                         T* h = reinterpret_cast<T*>(P.aux) + p * P.ld_aux;
@@ -865,7 +871,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                 constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
                 for (int it = 0; it < IT; ++it) {
-                    if (out_row[it] < 0 || n >= P.n) continue;
+                    if (!row_exists(mi, it) || n >= P.n) continue;
                     float u[PV], g[PV], d[PV], du[PV], dg[PV];
                     Elem<T>::unpack(to_uint4(hu[mi & 1][it]), u);
                     Elem<T>::unpack(to_uint4(hg[mi & 1][it]), g);
