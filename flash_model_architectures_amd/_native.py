@@ -89,6 +89,10 @@ PROTOTYPES: dict[str, tuple] = {
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int64, c_int, c_void_p],
     ),
+    "xma_scatter_rows_ordered": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p],
+    ),
     "xma_combine_topk": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int, c_void_p],

@@ -32,10 +32,13 @@ __global__ __launch_bounds__(256) void move_rows_vec_kernel(const T* __restrict_
     for (int64_t r0 = (int64_t)blockIdx.x * kRowsPerIter; r0 < rows; r0 += (int64_t)gridDim.x * kRowsPerIter) {
         int64_t srow[kRowsPerIter], drow[kRowsPerIter];
         float scale[kRowsPerIter];
+        bool live[kRowsPerIter];  // a gathered row whose index is negative has no source and is left as it is
 #pragma unroll
         for (int j = 0; j < kRowsPerIter; ++j) {
             const int64_t p = r0 + j < rows ? r0 + j : rows - 1;
-            const int64_t ix = index ? load_index(index, idx_is_i64, p) : p;
+            int64_t ix = index ? load_index(index, idx_is_i64, p) : p;
+            live[j] = r0 + j < rows && (MODE != kGather || ix >= 0);
+            if (MODE == kGather && ix < 0) ix = 0;
             srow[j] = MODE == kGather ? ix / fan_out : p;
             drow[j] = MODE == kGather ? p : ix;
             scale[j] = 1.0f;
@@ -55,7 +58,7 @@ __global__ __launch_bounds__(256) void move_rows_vec_kernel(const T* __restrict_
                     for (int q = 0; q < PV; ++q) f[q] *= scale[j];
                     v[j] = Elem<T>::pack(f);
                 }
-                if (r0 + j < rows) store_stream(dst + drow[j] * ld_dst + (int64_t)c * PV, v[j]);
+                if (live[j]) store_stream(dst + drow[j] * ld_dst + (int64_t)c * PV, v[j]);
             }
         }
     }
@@ -70,6 +73,7 @@ __global__ __launch_bounds__(256) void move_rows_scalar_kernel(const T* __restri
                                                                 const T* __restrict__ coeff) {
     for (int64_t p = blockIdx.x; p < rows; p += gridDim.x) {
         const int64_t ix = index ? load_index(index, idx_is_i64, p) : p;
+        if (MODE == kGather && ix < 0) continue;
         const int64_t srow = MODE == kGather ? ix / fan_out : p;
         const int64_t drow = MODE == kGather ? p : ix;
         float scale = 1.0f;
@@ -81,6 +85,20 @@ __global__ __launch_bounds__(256) void move_rows_scalar_kernel(const T* __restri
                 dst[drow * ld_dst + c] = src[srow * ld_src + c];
         }
     }
+}
+
+// inverse[index[p]] = p: who writes each destination row of a scatter (any one writer when several name the row;
+// -1, set beforehand, when nobody does).  Entries outside [0, dst_rows) are ignored.
+__global__ __launch_bounds__(256) void fill_minus_one_kernel(int32_t* __restrict__ inverse, int64_t dst_rows) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < dst_rows) inverse[i] = -1;
+}
+__global__ __launch_bounds__(256) void invert_index_kernel(const void* __restrict__ index, int idx_is_i64, int64_t rows,
+                                                           int64_t dst_rows, int32_t* __restrict__ inverse) {
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= rows) return;
+    const int64_t d = load_index(index, idx_is_i64, p);
+    if (d >= 0 && d < dst_rows) inverse[d] = (int32_t)p;
 }
 
 // y[t, :] = sum_j gates[t, j] * y_exp[t*k + j, :]   (GATED) or the plain sum over j.
@@ -239,6 +257,26 @@ int xma_scatter_rows(const void* src, int64_t ld_src, void* dst, int64_t ld_dst,
     XMA_DISPATCH_DTYPE(dtype, T, (launch_move<T, kScatter>(src, ld_src, dst, ld_dst, index, idx_is_i64, rows, cols, 1,
                                                            nullptr, (hipStream_t)stream_)))
     return check_launch("xma_scatter_rows");
+}
+
+int xma_scatter_rows_ordered(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, const void* index,
+                             int idx_is_i64, int64_t rows, int64_t dst_rows, int64_t cols, int dtype, void* inverse,
+                             void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    XMA_REQUIRE(valid_dtype(dtype), "xma_scatter_rows_ordered: bad dtype %d", dtype);
+    XMA_REQUIRE(rows >= 0 && dst_rows >= 0 && cols >= 0 && ld_src >= cols && ld_dst >= cols,
+                "xma_scatter_rows_ordered: bad shape");
+    XMA_REQUIRE(rows <= 0x7fffffff && dst_rows <= 0x7fffffff, "xma_scatter_rows_ordered: more than 2^31 - 1 rows");
+    if (rows == 0 || dst_rows == 0 || cols == 0) return 0;
+    XMA_REQUIRE(src && dst && index && inverse, "xma_scatter_rows_ordered: null pointer");
+    int32_t* inv = reinterpret_cast<int32_t*>(inverse);
+    hipLaunchKernelGGL(fill_minus_one_kernel, dim3((unsigned)ceil_div(dst_rows, 256)), dim3(256), 0, stream, inv,
+                       dst_rows);
+    hipLaunchKernelGGL(invert_index_kernel, dim3((unsigned)ceil_div(rows, 256)), dim3(256), 0, stream, index, idx_is_i64,
+                       rows, dst_rows, inv);
+    XMA_DISPATCH_DTYPE(dtype, T, (launch_move<T, kGather>(src, ld_src, dst, ld_dst, inv, 0, dst_rows, cols, 1, nullptr,
+                                                          stream)))
+    return check_launch("xma_scatter_rows_ordered");
 }
 
 int xma_combine_topk(const void* y_exp, int64_t ld_exp, const void* gates, void* y, int64_t ld_y, int64_t T,

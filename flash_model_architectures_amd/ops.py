@@ -238,13 +238,15 @@ def group(
 
 @xma_op(mutates_args={"out"})
 def ungroup(A: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> None:
-    """out[index[p]] = A[p]: the inverse row permutation of `group`."""
+    """out[index[p]] = A[p]: the inverse row permutation of `group`.  Rows of `out` that no index names keep
+    their contents; a row that several name receives one of them."""
 
     nat.require_device(A, index, out)
     assert A.dtype == out.dtype and A.size(1) == out.size(1) and A.size(0) == index.numel()
     index = index.contiguous()
+    inverse = _workspace(out.device, 4 * max(out.size(0), 1))
     nat.call(
-        "xma_scatter_rows",
+        "xma_scatter_rows_ordered",
         A.data_ptr(),
         _row_stride(A),
         out.data_ptr(),
@@ -252,9 +254,12 @@ def ungroup(A: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> None:
         index.data_ptr(),
         _i64(index),
         A.size(0),
+        out.size(0),
         A.size(1),
         nat.dtype_code(A),
+        inverse.data_ptr(),
         nat.stream(),
+        tag="xma_scatter_rows",
         nbytes=2 * A.numel() * A.element_size() + index.numel() * index.element_size(),
     )
 

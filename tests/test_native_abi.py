@@ -32,6 +32,7 @@ def test_header_declares_the_expected_entry_points():
         "xma_topk_softmax_bwd",
         "xma_gather_rows",
         "xma_scatter_rows",
+        "xma_scatter_rows_ordered",
         "xma_combine_topk",
         "xma_gate_grad",
         "xma_swiglu_forward",

@@ -29,6 +29,39 @@ def test_group_and_ungroup_are_exact(T, k, cols, dtype, idx_dtype):
     assert torch.equal(back.cpu(), want_back)
 
 
+@pytest.mark.parametrize("cols", [64, 37])
+def test_ungroup_partial_and_duplicate_targets(cols):
+    """The scatter runs in destination order through the inverted index: rows that no index names keep their
+    contents, a row that several name receives one of them whole, and the plain entry point of the library
+    (source order) gives the same result on a permutation."""
+
+    from flash_model_architectures_amd import _native as nat
+
+    g = torch.Generator().manual_seed(cols)
+    rows, dst_rows = 500, 800
+    src = torch.randn(rows, cols, generator=g)
+    index = torch.randperm(dst_rows, generator=g)[:rows].to(torch.int32)
+    index[10] = index[20] = index[30]  # one destination named three times
+    out = torch.full((dst_rows, cols), -7.0, device="cuda")
+    ops.ungroup(src.cuda(), index.cuda(), out)
+    out = out.cpu()
+    named = torch.zeros(dst_rows, dtype=torch.bool)
+    named[index.long()] = True
+    assert bool(torch.all(out[~named] == -7.0))
+    for p in range(rows):
+        if p not in (10, 20, 30):
+            assert torch.equal(out[index[p]], src[p])
+    assert any(torch.equal(out[index[30]], src[p]) for p in (10, 20, 30))
+
+    perm = torch.randperm(rows, generator=g).to(torch.int32).cuda()
+    a, b = torch.empty(rows, cols, device="cuda"), torch.empty(rows, cols, device="cuda")
+    ops.ungroup(src.cuda(), perm, a)
+    s = src.cuda()
+    nat.call("xma_scatter_rows", s.data_ptr(), s.stride(0), b.data_ptr(), b.stride(0), perm.data_ptr(), 0, rows, cols,
+             nat.dtype_code(s), nat.stream())
+    assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_group_with_coefficient(dtype):
     g = torch.Generator().manual_seed(2)
