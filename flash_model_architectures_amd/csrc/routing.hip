@@ -91,6 +91,9 @@ __global__ __launch_bounds__(256) void count_kernel(const IdT* __restrict__ ids,
 // every bin, so the output needs no clearing beforehand and the call is a single launch.
 constexpr int64_t kSingleBlockIds = (int64_t)1 << 15;  // most ids a single block is given (two chunks per wave)
 constexpr int kSingleBlockBins = 512;                  // most bins (16 replicas of 2 KiB in LDS)
+// The one-block counting sort also writes its output through a single compute unit, which moves some tens of bytes
+// per clock: beyond this size two launches over many blocks are faster.
+constexpr int64_t kSingleBlockSortIds = (int64_t)1 << 12;
 template <typename IdT>
 __global__ __launch_bounds__(1024) void count_single_block_kernel(const IdT* __restrict__ ids, int64_t n, int bins,
                                                                    uint32_t* __restrict__ counts) {
@@ -304,8 +307,111 @@ __global__ __launch_bounds__(256) void place_kernel(const IdT* __restrict__ ids,
         place_batch(v[j], begin + j * kWaveSize + lane, E, nbits, lane, next, sorted_ids, perm);
 }
 
-// The whole counting sort in ONE block of 16 waves, for up to kSingleBlockIds ids and kSingleBlockBins experts (the
-// routed rows of one MoE layer): wave w owns the w-th contiguous run of ids.  (1) every wave builds the histogram
+// Second and last launch of the counting sort for the sizes of an MoE layer (units * E <= kFusedScanValues, E <= 256;
+// the first launch is unit_hist_kernel).  One work-group moves data at a small fraction of the device's rate, so
+// the ids are spread over many small blocks, four waves = four units each, and every block repeats the scan for
+// itself: it reads the whole table of per-unit histograms (at most 64 KiB, L2-resident) and adds up, per expert,
+// all units (the expert's total) and the units before its own (where its ids start inside the expert's range);
+// thread e scans the totals into the offsets with wave shuffles; then every wave places the ids of its unit, which
+// it requested before the scan began.  Block 0 also writes counts and offsets.
+constexpr int kFusedScanValues = 16384;
+constexpr int kFusedUnitsPerBlock = 4;
+template <typename IdT, typename OutT>
+__global__ __launch_bounds__(256) void scan_place_kernel(const IdT* __restrict__ ids, int64_t n, int E, int nbits,
+                                                          int64_t units, const uint32_t* __restrict__ unit_hist,
+                                                          uint32_t* __restrict__ counts, int32_t* __restrict__ offsets,
+                                                          OutT* __restrict__ sorted_ids, OutT* __restrict__ perm) {
+    extern __shared__ uint32_t lds_hist[];  // total[E], before[E], next[4][E], wave_sum[4]
+    uint32_t* total = lds_hist;
+    uint32_t* before = lds_hist + E;
+    uint32_t* next_all = lds_hist + 2 * E;
+    uint32_t* wave_sum = lds_hist + (2 + kFusedUnitsPerBlock) * E;
+    const int wave = threadIdx.x / kWaveSize;
+    const int lane = lane_id();
+    const int64_t first_unit = (int64_t)blockIdx.x * kFusedUnitsPerBlock;
+
+    // this wave's ids, on their way while the scan runs
+    const int64_t begin = (first_unit + wave) * kChunk;
+    const int64_t end = begin + kChunk < n ? begin + kChunk : n;
+    int64_t v[kBatches];
+    load_chunk(ids, begin, end, lane, v);  // all -1 for a unit past the end
+
+    for (int i = threadIdx.x; i < 2 * E; i += 256) lds_hist[i] = 0;
+    __syncthreads();
+
+    // Thread (r, c) adds up column c (+ cols, + 2 cols ...) of the table over the units r, r + rows, ...; cols is E
+    // rounded up to a power of two, so consecutive lanes read consecutive words.
+    {
+        int cols = 1;
+        while (cols < E) cols <<= 1;
+        const int rows = 256 / cols;  // E <= 256
+        const int c = threadIdx.x & (cols - 1);
+        const int r = threadIdx.x / cols;
+        if (c < E) {
+            constexpr int kInFlight = 16;
+            uint32_t all = 0, mine = 0;
+            for (int64_t u0 = r; u0 < units; u0 += (int64_t)rows * kInFlight) {
+                uint32_t h[kInFlight];
+#pragma unroll
+                for (int j = 0; j < kInFlight; ++j) {
+                    const int64_t u = u0 + (int64_t)j * rows;
+                    h[j] = u < units ? unit_hist[u * E + c] : 0u;
+                }
+#pragma unroll
+                for (int j = 0; j < kInFlight; ++j) {
+                    const int64_t u = u0 + (int64_t)j * rows;
+                    all += h[j];
+                    mine += u < first_unit ? h[j] : 0u;
+                }
+            }
+            atomicAdd(&total[c], all);
+            atomicAdd(&before[c], mine);
+        }
+    }
+    __syncthreads();
+
+    // exclusive scan of the totals over the experts: thread e holds expert e
+    const int e = threadIdx.x;
+    const uint32_t count = e < E ? total[e] : 0u;
+    uint32_t inclusive = count;
+#pragma unroll
+    for (int d = 1; d < kWaveSize; d <<= 1) {
+        const uint32_t up = __shfl_up(inclusive, d, kWaveSize);
+        if (lane >= d) inclusive += up;
+    }
+    if (lane == kWaveSize - 1) wave_sum[wave] = inclusive;
+    __syncthreads();
+    uint32_t first_slot = inclusive - count;
+    for (int w = 0; w < wave; ++w) first_slot += wave_sum[w];
+    if (e < E) {
+        if (blockIdx.x == 0) {
+            counts[e] = count;
+            offsets[e] = (int32_t)first_slot;
+            if (e == E - 1) offsets[E] = (int32_t)(first_slot + count);
+        }
+        // first output slot of the ids of expert e in each of the block's units
+        uint32_t own[kFusedUnitsPerBlock];
+#pragma unroll
+        for (int w = 0; w < kFusedUnitsPerBlock; ++w)
+            own[w] = first_unit + w < units ? unit_hist[(first_unit + w) * E + e] : 0u;
+        uint32_t slot = first_slot + before[e];
+#pragma unroll
+        for (int w = 0; w < kFusedUnitsPerBlock; ++w) {
+            next_all[w * E + e] = slot;
+            slot += own[w];
+        }
+    }
+    __syncthreads();
+
+    if (begin >= n) return;
+    uint32_t* next = next_all + wave * E;
+#pragma unroll
+    for (int j = 0; j < kBatches; ++j)
+        place_batch(v[j], begin + j * kWaveSize + lane, E, nbits, lane, next, sorted_ids, perm);
+}
+
+// The whole counting sort in ONE block of 16 waves, for up to kSingleBlockSortIds ids and kSingleBlockBins experts (the
+// routed rows of a small batch): wave w owns the w-th contiguous run of ids.  (1) every wave builds the histogram
 // of its run in its own LDS row; (2) thread e turns column e into exclusive prefixes over the waves, the block
 // scans the column totals into the expert offsets, and the two are added up: row w, column e is then the first
 // output slot of wave w's ids of expert e; (3) every wave walks its run again in order and ranks equal ids inside
@@ -625,7 +731,7 @@ static int route_build_launch(const void* ids, int ids_is_i64, int64_t n, int32_
         return check_launch("xma_route_build");
     }
     const int nbits = ceil_log2(E);
-    if (n <= kSingleBlockIds && E <= kSingleBlockBins) {  // one launch, no workspace
+    if (n <= kSingleBlockSortIds && E <= kSingleBlockBins) {  // one launch, no workspace
         const size_t lds_one = ((size_t)E * (1024 / kWaveSize) + 1024) * sizeof(uint32_t);
 #define XMA_ROUTE_ONE(IdT, OutT)                                                                                     \
     hipLaunchKernelGGL((route_single_block_kernel<IdT, OutT>), dim3(1), dim3(1024), lds_one, stream, (const IdT*)ids, \
@@ -655,6 +761,27 @@ static int route_build_launch(const void* ids, int ids_is_i64, int64_t n, int32_
     else
         hipLaunchKernelGGL(unit_hist_kernel<int32_t>, dim3(blocks), dim3(wpb * kWaveSize), lds, stream,
                            (const int32_t*)ids, n, (int)E, wpb, unit_hist);
+    if (units * E <= kFusedScanValues && E <= 256) {  // second and last launch: scan and placement in one
+        const unsigned place_blocks = (unsigned)ceil_div(units, kFusedUnitsPerBlock);
+        const size_t place_lds = ((size_t)(2 + kFusedUnitsPerBlock) * E + kFusedUnitsPerBlock) * sizeof(uint32_t);
+#define XMA_SCAN_PLACE(IdT, OutT)                                                                                   \
+    hipLaunchKernelGGL((scan_place_kernel<IdT, OutT>), dim3(place_blocks), dim3(256), place_lds, stream,             \
+                       (const IdT*)ids, n, (int)E, nbits, units, (const uint32_t*)unit_hist, counts, offsets,       \
+                       (OutT*)sorted_ids, (OutT*)perm)
+        if (ids_is_i64) {
+            if (out_is_i64)
+                XMA_SCAN_PLACE(int64_t, int64_t);
+            else
+                XMA_SCAN_PLACE(int64_t, int32_t);
+        } else {
+            if (out_is_i64)
+                XMA_SCAN_PLACE(int32_t, int64_t);
+            else
+                XMA_SCAN_PLACE(int32_t, int32_t);
+        }
+#undef XMA_SCAN_PLACE
+        return check_launch("xma_route_build");
+    }
     hipLaunchKernelGGL(unit_scan_kernel, dim3((E + kWaveSize - 1) / kWaveSize), dim3(1024), 0, stream, unit_hist, units,
                        (int)E, counts);
     hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, stream, (const uint32_t*)counts, (int)E, offsets);
