@@ -741,28 +741,33 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
                     }
             }
         }
-        auto write_rows = [&](char* buf, const f32x16_t (&a)[NI]) {
+        // (the bias is a copy of the code of its own: a wave alone on its SIMD pays for every instruction, and as
+        // one copy the compiler adds a selected zero to every sum of a launch that has no bias)
+        auto write_rows = [&](char* buf, const f32x16_t (&a)[NI], auto bias_tag) {
+            constexpr bool BIAS = decltype(bias_tag)::value;
 #pragma unroll
             for (int ni = 0; ni < NI; ++ni) {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const int chunk = ((wn0 + ni * 32 + 8 * g) >> 3) ^ (br & 31);
                     float v[4] = {a[ni][4 * g], a[ni][4 * g + 1], a[ni][4 * g + 2], a[ni][4 * g + 3]};
-                    if constexpr (KIND == XMA_GEMM_TN) {
-                        if (with_bias) {
+                    if constexpr (BIAS) {
 #pragma unroll
-                            for (int q = 0; q < 4; ++q) v[q] += bias[ni][g][q];
-                        }
+                        for (int q = 0; q < 4; ++q) v[q] += bias[KIND == XMA_GEMM_TN ? ni : 0][KIND == XMA_GEMM_TN ? g : 0][KIND == XMA_GEMM_TN ? q : 0];
                     }
                     *reinterpret_cast<uint2*>(buf + br * (BN * 2) + (chunk << 4) + half * 8) =
                         make_uint2(Elem<T>::pack2(v[0], v[1]), Elem<T>::pack2(v[2], v[3]));
                 }
             }
         };
-        write_rows(slab<0>(), acc[0]);
-        write_rows(slab<1>(), acc[1]);
-        write_rows(slab<2>(), acc[2]);
-        write_rows(slab<3>(), acc[3]);
+        auto write_all = [&](auto bias_tag) {
+            write_rows(slab<0>(), acc[0], bias_tag);
+            write_rows(slab<1>(), acc[1], bias_tag);
+            write_rows(slab<2>(), acc[2], bias_tag);
+            write_rows(slab<3>(), acc[3], bias_tag);
+        };
+        if (KIND == XMA_GEMM_TN && with_bias) write_all(std::true_type{});
+        else write_all(std::false_type{});
     }
     __syncthreads();
 
