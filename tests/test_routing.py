@@ -28,7 +28,7 @@ def _check_route(ids: torch.Tensor, E: int, index_dtype=torch.int32):
 
 
 @pytest.mark.parametrize("n,E", [(1, 1), (2, 8), (14, 8), (63, 2), (64, 2), (65, 3), (1023, 8), (1024, 8), (1025, 8),
-                                 (4096, 64), (4097, 8), (16384, 8), (98304, 64), (131072, 128), (65536, 256), (70000, 200),
+                                 (4096, 64), (4097, 8), (16384, 8), (32768, 256), (20000, 37), (32769, 8), (5001, 1), (98304, 64), (131072, 128), (65536, 256), (70000, 200),
                                  (66000, 256), (5000, 1000), (20000, 16384)])
 @pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
 def test_route_matches_oracle(n, E, dtype):
