@@ -55,6 +55,66 @@ def test_swiglu_packed(size, dtype):
     assert_close(xd.grad, xo.grad, TOL[dtype], "dx")
 
 
+def _reference_size_matrix():
+    """The size scheme of the reference's swiglu test (tests/test_commons.py:49-61 as used by
+    tests/functional/swiglu_test.py:15-22): squares (2^i + j)^2 for i < 15, j < 10, and 50 rectangles with both sides
+    drawn from 3000 +- 1000; drawn here from a fixed seed."""
+
+    import random
+
+    rng = random.Random(0)
+    sizes = {(2**i + j, 2**i + j) for i in range(15) for j in range(10)}
+    sizes |= {(3000 + rng.randint(-1000, 1000), 3000 + rng.randint(-1000, 1000)) for _ in range(50)}
+    return sorted(sizes)
+
+
+def _close_on_device(got, want, tol, what):
+    """The two checks of helpers.assert_close, evaluated where the tensors live (the largest sizes of the matrix
+    hold 2.7e8 elements)."""
+
+    g, w = got.detach().float(), want.detach().float()
+    scale = w.abs().max().item()
+    err = (g - w).abs().max().item() / (scale if scale > 0 else 1.0)
+    assert err <= tol, f"{what}: max relative error {err:.3e} > {tol:.1e}"
+    rms = w.double().pow(2).mean().sqrt().item()
+    if rms > 0:
+        elem = ((g - w).abs() / (w.abs() + rms)).max().item()
+        assert elem <= 2 * tol, f"{what}: element-wise error {elem:.3e} > {2 * tol:.1e}"
+    else:
+        assert not bool(g.any()), f"{what}: expected exact zeros"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_swiglu_reference_size_matrix(dtype):
+    """Every size of the reference's matrix (odd widths included: no rounding up to 16 bytes), forward and the
+    backward of a mean (fp32) or a sum (16-bit types), against the
+    oracle's formula evaluated by torch in fp32 on the same device tensors.  The reference's own bars for fp32
+    (atol 5.4e-5 forward, 5e-6 on the gradients, rtol 0, tests/functional/swiglu_test.py:56-62) are checked on top
+    of this build's."""
+
+    torch.manual_seed(0)
+    for rows, cols in _reference_size_matrix():
+        gate = (torch.randn(rows, cols, device="cuda") * 2).to(dtype).requires_grad_()
+        up = torch.randn(rows, cols, device="cuda").to(dtype).requires_grad_()
+        # fp32: the gradient of a mean, as in the reference's test; 16-bit types: of a sum (1 / numel and everything
+        # multiplied by it fall into the subnormal range of fp16 from 2^14 elements on, where relative bars mean nothing)
+        dy = torch.full((rows, cols), 1.0 / (rows * cols) if dtype == torch.float32 else 1.0, device="cuda").to(dtype)
+        y = xma.swiglu(gate, up, kernel_backend=xma.KernelBackend.rocm)
+        y.backward(dy)
+        go, uo = gate.detach().float().requires_grad_(), up.detach().float().requires_grad_()
+        yo = to.swiglu(go, uo)
+        yo.backward(dy.float())
+        what = f"{rows}x{cols}"
+        _close_on_device(y, yo, TOL[dtype], "y " + what)
+        _close_on_device(gate.grad, go.grad, TOL[dtype], "d_gate " + what)
+        _close_on_device(up.grad, uo.grad, TOL[dtype], "d_up " + what)
+        if dtype == torch.float32:
+            assert (y - yo).abs().max().item() <= 5.4e-5, what
+            assert (gate.grad - go.grad).abs().max().item() <= 5e-6, what
+            assert (up.grad - uo.grad).abs().max().item() <= 5e-6, what
+        del gate, up, dy, y, go, uo, yo
+
+
 def test_swiglu_keeps_leading_dims_and_accepts_views():
     x = torch.randn(3, 5, 7, 32)
     y = xma.swiglu_packed(x.cuda())
