@@ -197,9 +197,9 @@ __device__ __forceinline__ bool locate_tile(int row_tiles, int col_tiles, int& r
 // for a whole tile time, so each of them is cut along the reduction into S = min(kMaxSplit, C / R,
 // stages / kSplitMinStages) parts that run side by side.  Only when the launch has fewer than kSplitMaxRounds
 // rounds (the idle units of a last round matter less the more rounds there are), and only while a part keeps
-// kSplitMinStages stages: every part parks a 256 KiB tile of fp32 sums in HBM and the last one reads them all
-// back, which costs about as much as 16 stages of the main loop (measured: reductions of 2048 split in two lose
-// 20 % of the launch, reductions of 14336 split in three gain 8 %).  Work-groups are dealt per XCD as in
+// kSplitMinStages stages: every part parks a 256 KiB tile of fp32 sums in memory and the last one reads them all
+// back, 40-50 k cycles or about 17 stages of the main loop (measured; reductions of 14336 and 28672 split in three
+// gain 7 % and 5 % of their launches).  Work-groups are dealt per XCD as in
 // locate_tile<false>: XCD x takes the x-th eighth of the whole tiles, then the x-th eighth of the parts
 // (part-major, so neighbours share panels).
 struct TileWork {

@@ -583,49 +583,71 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     // (so the result does not depend on the arrival order) and goes on to the epilogue ----
     if constexpr (KIND != XMA_GEMM_MT) {
         if (work.parts > 1) {
-            typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+            // The parts of a tile run on different XCDs, whose L2 caches are not kept coherent with each other.  Fences
+            // at device scope would do (each writes back and invalidates the XCD's whole L2, once per wave, under
+            // every other work-group of the XCD: 150-200 k cycles per exchange, measured); instead the partial sums
+            // and the arrival counter are accessed with relaxed device-scope atomics, which go through to memory by
+            // themselves, and what orders them is that every wave's stores have completed before the barrier that
+            // precedes the arrival.
             auto part_buffer = [&](int part) {
-                return reinterpret_cast<f32x4_t*>(P.split_partials +
-                                                  (int64_t)(part * work.split_tiles + work.split_tile) * kSplitTileFloats);
+                return reinterpret_cast<uint64_t*>(P.split_partials +
+                                                   (int64_t)(part * work.split_tiles + work.split_tile) * kSplitTileFloats);
             };
-            f32x4_t* mine = part_buffer(work.part);
+            uint64_t* mine = part_buffer(work.part);
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-                    for (int g = 0; g < 4; ++g)
-                        mine[((mi * NI + ni) * 4 + g) * THREADS + tid] =
-                            f32x4_t{acc[mi][ni][4 * g], acc[mi][ni][4 * g + 1], acc[mi][ni][4 * g + 2], acc[mi][ni][4 * g + 3]};
-            __threadfence();  // this thread's partial sums are visible to the whole device ...
-            __syncthreads();  // ... and so are everybody else's, before the arrival is counted
+                    for (int g = 0; g < 8; ++g) {
+                        const float2 v{acc[mi][ni][2 * g], acc[mi][ni][2 * g + 1]};
+                        __hip_atomic_store(mine + ((mi * NI + ni) * 8 + g) * THREADS + tid, __builtin_bit_cast(uint64_t, v),
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+            wait_vmcnt<0>();  // this wave's partial sums have reached memory ...
+            __syncthreads();  // ... and so have everybody else's, before the arrival is counted
             int* arrivals = reinterpret_cast<int*>(slab<0>());
             if (tid == 0)
-                arrivals[0] = __hip_atomic_fetch_add(P.split_counters + work.split_tile, 1, __ATOMIC_ACQ_REL,
+                arrivals[0] = __hip_atomic_fetch_add(P.split_counters + work.split_tile, 1, __ATOMIC_RELAXED,
                                                      __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
             const bool last = arrivals[0] == work.parts - 1;
             __syncthreads();  // the slab is reused below
             if (!last) return;
-            __threadfence();
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
+            // The sums are requested 32 loads at a time and added afterwards: with all 256 accumulators live the
+            // compiler otherwise fetches them one by one, a full memory latency each.
             for (int part = 0; part < work.parts; ++part) {
-                const f32x4_t* src = part_buffer(part);
+                const uint64_t* src = part_buffer(part);
 #pragma unroll
-                for (int mi = 0; mi < MI; ++mi)
+                for (int mi = 0; mi < MI; ++mi) {
+                    uint64_t v[NI][8];
 #pragma unroll
                     for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-                        for (int g = 0; g < 4; ++g) {
-                            const f32x4_t v = src[((mi * NI + ni) * 4 + g) * THREADS + tid];
+                        for (int g = 0; g < 8; ++g)
+                            v[ni][g] = __hip_atomic_load(src + ((mi * NI + ni) * 8 + g) * THREADS + tid, __ATOMIC_RELAXED,
+                                                         __HIP_MEMORY_SCOPE_AGENT);
+                    batch_fence();
 #pragma unroll
-                            for (int q = 0; q < 4; ++q) acc[mi][ni][4 * g + q] += v[q];
+                    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                        for (int g = 0; g < 8; ++g) pin(v[ni][g]);
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                        for (int g = 0; g < 8; ++g) {
+                            const float2 f = __builtin_bit_cast(float2, v[ni][g]);
+                            acc[mi][ni][2 * g] += f.x;
+                            acc[mi][ni][2 * g + 1] += f.y;
                         }
+                    batch_fence();
+                }
             }
         }
     }

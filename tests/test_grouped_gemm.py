@@ -219,35 +219,44 @@ def test_ragged_tail_rows_are_not_touched():
     assert_close(out, ref, TOL[torch.bfloat16])
 
 
+@pytest.mark.parametrize("K", [4160, 6200, 8320])
 @pytest.mark.parametrize("layout", ["TN", "NN"])
-def test_whole_rounds_plus_split_remainder(layout):
+def test_whole_rounds_plus_split_remainder(layout, K):
     """More tiles than compute units, with a remainder: the first tiles run whole, the tiles of the last,
     partly filled round are reduced in parts and summed by the part that finishes last (a part keeps at least 32
-    stages of 64, so the reduction must be long: 6200 = 96 stages and a tail, cut in three).  Checked against fp32
-    matmuls on the device; run twice to see that the result does not depend on the arrival order."""
+    stages of 64, so the reduction must be long: 4160 is cut in two, 6200 = 96 stages and a tail in three, 8320 in
+    four).  The parts hand their sums over through memory that the next launch reuses, so two operand sets are run
+    alternately, several times: every result must equal the fp32 matmuls on the device within the bar, and all
+    results of one operand set must be bit-identical (the sum does not depend on the arrival order, and nothing of
+    the other set's sums may be picked up)."""
 
     dev = "cuda"
-    E, K, N = 4, 6200, 1792  # 7 column tiles; ~43 row tiles -> ~300 tiles on 256 compute units
+    E, N = 4, 1792  # 7 column tiles; ~43 row tiles -> ~300 tiles on 256 compute units
     sizes = [2700, 1, 3100, 4300]
     M = sum(sizes)
-    g = torch.Generator().manual_seed(3)
-    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
-    w = (torch.randn(E, N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)  # [E, N, K]
+    g = torch.Generator().manual_seed(3 + K)
     off = torch.tensor([0] + list(torch.tensor(sizes).cumsum(0)), dtype=torch.int32, device=dev)
     idx = torch.arange(M, dtype=torch.int32, device=dev)
     se = torch.repeat_interleave(torch.arange(E), torch.tensor(sizes)).int().to(dev)
-    if layout == "TN":
-        weights = w.permute(0, 2, 1)  # logical [E, K, N], K contiguous
-    else:
-        weights = w.permute(0, 2, 1).contiguous()  # [E, K, N], N contiguous
-    outs = []
+    sets = []
     for _ in range(2):
-        out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
-        ops.scatter2scatter(a, weights, se, idx, out, 1, True, True, off)
-        outs.append(out)
-    ref = torch.cat([a[off[e] : off[e + 1]].float() @ w[e].float().T for e in range(E)])
-    assert_close(outs[0], ref, TOL[torch.bfloat16])
-    assert torch.equal(outs[0], outs[1])
+        a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+        w = (torch.randn(E, N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)  # [E, N, K]
+        if layout == "TN":
+            weights = w.permute(0, 2, 1)  # logical [E, K, N], K contiguous
+        else:
+            weights = w.permute(0, 2, 1).contiguous()  # [E, K, N], N contiguous
+        ref = torch.cat([a[off[e] : off[e + 1]].float() @ w[e].float().T for e in range(E)])
+        sets.append((a, weights, ref, []))
+    for _ in range(3):
+        for a, weights, ref, outs in sets:
+            out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+            ops.scatter2scatter(a, weights, se, idx, out, 1, True, True, off)
+            outs.append(out)
+    for a, weights, ref, outs in sets:
+        assert_close(outs[0], ref, TOL[torch.bfloat16])
+        for out in outs[1:]:
+            assert torch.equal(outs[0], out)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
