@@ -690,11 +690,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
                 for (int it = 0; it < IT; ++it) orow[mi][it] = index_of(safe_row(mi, it));
-            batch_fence();
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-                for (int it = 0; it < IT; ++it) pin(orow[mi][it]);
+            batch_fence();  // the loads stay in flight while the accumulators are packed; they are waited for after that
         };
         if (EPI == EPI_BACKWARD || P.out_index == nullptr) {  // that epilogue only writes grouped rows
             const int32_t first = (int32_t)m_begin;
@@ -790,6 +786,13 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         };
         if (KIND == XMA_GEMM_TN && with_bias) write_all(std::true_type{});
         else write_all(std::false_type{});
+    }
+    if constexpr (KIND != XMA_GEMM_MT) {
+        batch_fence();
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int it = 0; it < IT; ++it) pin(orow[mi][it]);
     }
     __syncthreads();
 
