@@ -116,6 +116,24 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y_ex
             for (int q = 0; q < PV; ++q) acc[q] = 0.0f;
             int j = 0;
             if constexpr (VEC) {
+                // four rows in flight per thread while there are four, then two: the walk over a token's k rows
+                // is otherwise a chain of load latencies
+                for (; j + 4 <= k; j += 4) {
+                    uint4 v[4];
+                    float g[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        v[r] = *reinterpret_cast<const uint4*>(base + (int64_t)(j + r) * ld_exp + c * PV);
+                        g[r] = GATED ? Elem<T>::load(gates + t * k + j + r) : 1.0f;
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float f[PV];
+                        Elem<T>::unpack(v[r], f);
+#pragma unroll
+                        for (int q = 0; q < PV; ++q) acc[q] = fmaf(g[r], f[q], acc[q]);
+                    }
+                }
                 for (; j + 2 <= k; j += 2) {
                     const uint4 v0 = *reinterpret_cast<const uint4*>(base + (int64_t)j * ld_exp + c * PV);
                     const uint4 v1 = *reinterpret_cast<const uint4*>(base + (int64_t)(j + 1) * ld_exp + c * PV);
@@ -152,7 +170,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y_ex
 
 // d_gates[t, j] = <y_exp[t*k + j, :], dy[t, :]>; block per token, wave per slot j.
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void gate_grad_kernel(const T* __restrict__ y_exp, int64_t ld_exp,
+__global__ __launch_bounds__(1024) void gate_grad_kernel(const T* __restrict__ y_exp, int64_t ld_exp,
                                                          const T* __restrict__ dy, int64_t ld_dy,
                                                          T* __restrict__ d_gates, int64_t Tn, int k, int64_t cols) {
     constexpr int PV = VEC ? Elem<T>::kPerVec : 1;
@@ -165,7 +183,27 @@ __global__ __launch_bounds__(256) void gate_grad_kernel(const T* __restrict__ y_
             const T* row = y_exp + (t * k + j) * ld_exp;
             const T* g = dy + t * ld_dy;
             float acc = 0.0f;
-            for (int64_t c = lane; c < chunks; c += kWaveSize) {
+            int64_t c = lane;
+            if constexpr (VEC) {
+                // four chunk pairs in flight per lane
+                for (; c + 3 * kWaveSize < chunks; c += 4 * kWaveSize) {
+                    uint4 ra[4], rb[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        ra[r] = *reinterpret_cast<const uint4*>(row + (c + r * kWaveSize) * PV);
+                        rb[r] = *reinterpret_cast<const uint4*>(g + (c + r * kWaveSize) * PV);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float a[PV], b[PV];
+                        Elem<T>::unpack(ra[r], a);
+                        Elem<T>::unpack(rb[r], b);
+#pragma unroll
+                        for (int q = 0; q < PV; ++q) acc = fmaf(a[q], b[q], acc);
+                    }
+                }
+            }
+            for (; c < chunks; c += kWaveSize) {
                 if constexpr (VEC) {
                     float a[PV], b[PV];
                     Elem<T>::unpack(*reinterpret_cast<const uint4*>(row + c * PV), a);
@@ -317,7 +355,8 @@ int xma_gate_grad(const void* y_exp, int64_t ld_exp, const void* dy, int64_t ld_
     XMA_REQUIRE(y_exp && dy && d_gates, "xma_gate_grad: null pointer");
     XMA_DISPATCH_DTYPE(
         dtype, T_, const bool vec = vec_ok<T_>(y_exp, ld_exp, dy, ld_dy, cols);
-        const dim3 grid(row_grid(T)), block(256);
+        // one wave per slot of the token's k, so that no wave of the block idles
+        const dim3 grid(row_grid(T)), block((unsigned)(kWaveSize * (k < 16 ? k : 16)));
         if (vec) hipLaunchKernelGGL((gate_grad_kernel<T_, true>), grid, block, 0, stream, (const T_*)y_exp, ld_exp,
                                     (const T_*)dy, ld_dy, (T_*)d_gates, T, (int)k, cols);
         else hipLaunchKernelGGL((gate_grad_kernel<T_, false>), grid, block, 0, stream, (const T_*)y_exp, ld_exp,
