@@ -28,11 +28,11 @@ __global__ __launch_bounds__(256) void add_expert_bias_kernel(T* __restrict__ y,
         for (int64_t c = cl; c < chunks; c += 32) {
             if constexpr (VEC) {
                 float a[PV], v[PV];
-                Elem<T>::unpack(*reinterpret_cast<const uint4*>(row + c * PV), a);
+                Elem<T>::unpack(load_stream(row + c * PV), a);
                 Elem<T>::unpack(*reinterpret_cast<const uint4*>(b + c * PV), v);
 #pragma unroll
                 for (int q = 0; q < PV; ++q) a[q] += v[q];
-                *reinterpret_cast<uint4*>(row + c * PV) = Elem<T>::pack(a);
+                store_stream(row + c * PV, Elem<T>::pack(a));
             } else {
                 Elem<T>::store(row + c, Elem<T>::load(row + c) + Elem<T>::load(b + c));
             }
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(1024) void expert_colsum_kernel(const T* __restrict
         for (int64_t r = begin + rl; r < end; r += 32) {
             if constexpr (VEC) {
                 float a[PV];
-                Elem<T>::unpack(*reinterpret_cast<const uint4*>(src + r * ld + chunk * PV), a);
+                Elem<T>::unpack(load_stream(src + r * ld + chunk * PV), a);
 #pragma unroll
                 for (int q = 0; q < PV; ++q) acc[q] += a[q];
             } else {

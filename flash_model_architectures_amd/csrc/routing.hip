@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) void count_kernel(const IdT* __restrict__ ids,
         const int64_t nvec = n / kPerVec;
         const uint4* v = reinterpret_cast<const uint4*>(ids);
         for (int64_t i = tid; i < nvec; i += nthreads) {
-            uint4 q = v[i];
+            uint4 q = load_stream(v + i);
             IdT e[kPerVec];
             if constexpr (sizeof(IdT) == 4) {
                 e[0] = (IdT)q.x;

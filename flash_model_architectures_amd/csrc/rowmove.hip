@@ -10,16 +10,9 @@ constexpr int kRowsPerIter = 1;
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
-// Streaming accesses: each byte is touched once, so keep it from displacing reusable lines in the caches.
-__device__ __forceinline__ uint4 load_stream(const void* p) {
-    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
-    return make_uint4(v.x, v.y, v.z, v.w);
-}
-__device__ __forceinline__ void store_stream(void* p, const uint4& v) {
-    __builtin_nontemporal_store(u32x4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4_t*>(p));
-}
-
 enum RowMode { kGather = 0, kScatter = 1 };
+
+constexpr int64_t kInfinityCacheBytes = (int64_t)256 << 20;
 
 // 16-byte path: cols is a multiple of Elem<T>::kPerVec, strides keep rows 16-byte aligned.
 template <typename T, int MODE, bool COEFF>
@@ -102,12 +95,19 @@ __global__ __launch_bounds__(256) void invert_index_kernel(const void* __restric
 }
 
 // y[t, :] = sum_j gates[t, j] * y_exp[t*k + j, :]   (GATED) or the plain sum over j.
-template <typename T, bool GATED, bool VEC>
+// STREAM: the expanded rows are read with streaming loads.  That is the faster way when they come from HBM; rows that
+// the previous kernel has just written and that fit the 256 MiB Infinity Cache are served from there, and plain
+// loads are faster (measured: 34 vs 37 us on 128 MiB of rows).
+template <typename T, bool GATED, bool VEC, bool STREAM>
 __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y_exp, int64_t ld_exp,
                                                        const T* __restrict__ gates, T* __restrict__ y, int64_t ld_y,
                                                        int64_t Tn, int k, int64_t cols) {
     constexpr int PV = VEC ? Elem<T>::kPerVec : 1;
     const int64_t chunks = cols / PV;
+    auto load_row_chunk = [](const T* p) {
+        if constexpr (STREAM) return load_stream(p);
+        else return *reinterpret_cast<const uint4*>(p);
+    };
     for (int64_t t = blockIdx.x; t < Tn; t += gridDim.x) {
         const T* base = y_exp + t * k * ld_exp;
         for (int64_t c = threadIdx.x; c < chunks; c += blockDim.x) {
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y_ex
                     float g[4];
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        v[r] = *reinterpret_cast<const uint4*>(base + (int64_t)(j + r) * ld_exp + c * PV);
+                        v[r] = load_row_chunk(base + (int64_t)(j + r) * ld_exp + c * PV);
                         g[r] = GATED ? Elem<T>::load(gates + t * k + j + r) : 1.0f;
                     }
 #pragma unroll
@@ -135,8 +135,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y_ex
                     }
                 }
                 for (; j + 2 <= k; j += 2) {
-                    const uint4 v0 = *reinterpret_cast<const uint4*>(base + (int64_t)j * ld_exp + c * PV);
-                    const uint4 v1 = *reinterpret_cast<const uint4*>(base + (int64_t)(j + 1) * ld_exp + c * PV);
+                    const uint4 v0 = load_row_chunk(base + (int64_t)j * ld_exp + c * PV);
+                    const uint4 v1 = load_row_chunk(base + (int64_t)(j + 1) * ld_exp + c * PV);
                     float f0[PV], f1[PV];
                     Elem<T>::unpack(v0, f0);
                     Elem<T>::unpack(v1, f1);
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y_ex
             for (; j < k; ++j) {
                 const float g = GATED ? Elem<T>::load(gates + t * k + j) : 1.0f;
                 if constexpr (VEC) {
-                    const uint4 v = *reinterpret_cast<const uint4*>(base + (int64_t)j * ld_exp + c * PV);
+                    const uint4 v = load_row_chunk(base + (int64_t)j * ld_exp + c * PV);
                     float f[PV];
                     Elem<T>::unpack(v, f);
 #pragma unroll
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(1024) void gate_grad_kernel(const T* __restrict__ y
                     uint4 ra[4], rb[4];
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        ra[r] = *reinterpret_cast<const uint4*>(row + (c + r * kWaveSize) * PV);
+                        ra[r] = load_stream(row + (c + r * kWaveSize) * PV);
                         rb[r] = *reinterpret_cast<const uint4*>(g + (c + r * kWaveSize) * PV);
                     }
 #pragma unroll
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(1024) void gate_grad_kernel(const T* __restrict__ y
             for (; c < chunks; c += kWaveSize) {
                 if constexpr (VEC) {
                     float a[PV], b[PV];
-                    Elem<T>::unpack(*reinterpret_cast<const uint4*>(row + c * PV), a);
+                    Elem<T>::unpack(load_stream(row + c * PV), a);
                     Elem<T>::unpack(*reinterpret_cast<const uint4*>(g + c * PV), b);
 #pragma unroll
                     for (int q = 0; q < PV; ++q) acc = fmaf(a[q], b[q], acc);
@@ -324,11 +324,18 @@ int xma_combine_topk(const void* y_exp, int64_t ld_exp, const void* gates, void*
     XMA_REQUIRE(T >= 0 && k >= 1 && cols >= 0 && ld_exp >= cols && ld_y >= cols, "xma_combine_topk: bad shape");
     if (T == 0 || cols == 0) return 0;
     XMA_REQUIRE(y_exp && y, "xma_combine_topk: null pointer");
-#define XMA_COMBINE(G, V)                                                                           \
-    hipLaunchKernelGGL((combine_kernel<T_, G, V>), grid, block, 0, stream, (const T_*)y_exp, ld_exp, \
-                       (const T_*)gates, (T_*)y, ld_y, T, (int)k, cols)
+#define XMA_COMBINE(G, V)                                                                                         \
+    do {                                                                                                          \
+        if (from_hbm)                                                                                             \
+            hipLaunchKernelGGL((combine_kernel<T_, G, V, true>), grid, block, 0, stream, (const T_*)y_exp, ld_exp, \
+                               (const T_*)gates, (T_*)y, ld_y, T, (int)k, cols);                                   \
+        else                                                                                                      \
+            hipLaunchKernelGGL((combine_kernel<T_, G, V, false>), grid, block, 0, stream, (const T_*)y_exp,       \
+                               ld_exp, (const T_*)gates, (T_*)y, ld_y, T, (int)k, cols);                           \
+    } while (0)
     XMA_DISPATCH_DTYPE(
         dtype, T_, const bool vec = vec_ok<T_>(y_exp, ld_exp, y, ld_y, cols);
+        const bool from_hbm = T * k * cols * (int64_t)sizeof(T_) > kInfinityCacheBytes;
         const int64_t chunks = vec ? cols / Elem<T_>::kPerVec : cols;
         const dim3 grid(row_grid(T)), block(row_block(chunks));
         if (gates) {

@@ -31,8 +31,8 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const T* __restrict__ g
 #pragma unroll
             for (int j = 0; j < kRowUnroll; ++j) {
                 const int64_t r = r0 + j * row_step < rows ? r0 + j * row_step : r0;
-                gv[j] = *reinterpret_cast<const uint4*>(gate + r * ld_g + c * PV);
-                uv[j] = *reinterpret_cast<const uint4*>(up + r * ld_u + c * PV);
+                gv[j] = load_stream(gate + r * ld_g + c * PV);
+                uv[j] = load_stream(up + r * ld_u + c * PV);
             }
 #pragma unroll
             for (int j = 0; j < kRowUnroll; ++j) {
@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const T* __restrict__ g
                 Elem<T>::unpack(uv[j], u);
 #pragma unroll
                 for (int q = 0; q < PV; ++q) o[q] = swiglu_f(g[q], u[q]);
-                *reinterpret_cast<uint4*>(y + r * ld_y + c * PV) = Elem<T>::pack(o);
+                store_stream(y + r * ld_y + c * PV, Elem<T>::pack(o));
             }
         } else {
 #pragma unroll
@@ -73,9 +73,9 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ g
 #pragma unroll
             for (int j = 0; j < kRowUnroll; ++j) {
                 const int64_t r = r0 + j * row_step < rows ? r0 + j * row_step : r0;
-                gv[j] = *reinterpret_cast<const uint4*>(gate + r * ld_g + c * PV);
-                uv[j] = *reinterpret_cast<const uint4*>(up + r * ld_u + c * PV);
-                dv[j] = *reinterpret_cast<const uint4*>(dy + r * ld_dy + c * PV);
+                gv[j] = load_stream(gate + r * ld_g + c * PV);
+                uv[j] = load_stream(up + r * ld_u + c * PV);
+                dv[j] = load_stream(dy + r * ld_dy + c * PV);
             }
 #pragma unroll
             for (int j = 0; j < kRowUnroll; ++j) {
@@ -87,8 +87,8 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ g
                 Elem<T>::unpack(dv[j], d);
 #pragma unroll
                 for (int q = 0; q < PV; ++q) swiglu_b(g[q], u[q], d[q], og[q], ou[q]);
-                *reinterpret_cast<uint4*>(dgate + r * ld_dg + c * PV) = Elem<T>::pack(og);
-                *reinterpret_cast<uint4*>(dup + r * ld_du + c * PV) = Elem<T>::pack(ou);
+                store_stream(dgate + r * ld_dg + c * PV, Elem<T>::pack(og));
+                store_stream(dup + r * ld_du + c * PV, Elem<T>::pack(ou));
             }
         } else {
 #pragma unroll
