@@ -37,23 +37,34 @@ __global__ __launch_bounds__(256) void move_rows_vec_kernel(const T* __restrict_
             scale[j] = 1.0f;
             if constexpr (COEFF) scale[j] = Elem<T>::load(coeff + ix);
         }
-        for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
-            uint4 v[kRowsPerIter];
+        // kChunksInFlight chunks of each row requested before the first is stored
+        constexpr int kChunksInFlight = 2;
+        auto move = [&](int c0, int count) {
+            uint4 v[kChunksInFlight][kRowsPerIter];
 #pragma unroll
-            for (int j = 0; j < kRowsPerIter; ++j)
-                v[j] = load_stream(src + srow[j] * ld_src + (int64_t)c * PV);
+            for (int i = 0; i < kChunksInFlight; ++i)
 #pragma unroll
-            for (int j = 0; j < kRowsPerIter; ++j) {
-                if constexpr (COEFF) {
-                    float f[PV];
-                    Elem<T>::unpack(v[j], f);
+                for (int j = 0; j < kRowsPerIter; ++j)
+                    if (i < count) v[i][j] = load_stream(src + srow[j] * ld_src + (int64_t)(c0 + i * (int)blockDim.x) * PV);
 #pragma unroll
-                    for (int q = 0; q < PV; ++q) f[q] *= scale[j];
-                    v[j] = Elem<T>::pack(f);
+            for (int i = 0; i < kChunksInFlight; ++i)
+#pragma unroll
+                for (int j = 0; j < kRowsPerIter; ++j) {
+                    if (i >= count) continue;
+                    if constexpr (COEFF) {
+                        float f[PV];
+                        Elem<T>::unpack(v[i][j], f);
+#pragma unroll
+                        for (int q = 0; q < PV; ++q) f[q] *= scale[j];
+                        v[i][j] = Elem<T>::pack(f);
+                    }
+                    if (live[j]) store_stream(dst + drow[j] * ld_dst + (int64_t)(c0 + i * (int)blockDim.x) * PV, v[i][j]);
                 }
-                if (live[j]) store_stream(dst + drow[j] * ld_dst + (int64_t)c * PV, v[j]);
-            }
-        }
+        };
+        int c = threadIdx.x;
+        for (; c + (kChunksInFlight - 1) * (int)blockDim.x < chunks; c += kChunksInFlight * (int)blockDim.x)
+            move(c, kChunksInFlight);
+        for (; c < chunks; c += blockDim.x) move(c, 1);
     }
 }
 
