@@ -716,8 +716,8 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
             const T* h = reinterpret_cast<const T*>(P.aux) + (m_begin + safe_row(mi, it)) * P.ld_aux;
-            up[it] = *reinterpret_cast<const u32x4_t*>(h + n);
-            gate[it] = *reinterpret_cast<const u32x4_t*>(h + second_half + n);
+            up[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(h + n));
+            gate[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(h + second_half + n));
         }
     };
     if constexpr (SWBWD) load_saved(0, hu[0], hg[0]);
