@@ -655,8 +655,8 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     // ---- epilogue: accumulators -> LDS (slab mi holds the 64 tile rows {wr*128 + mi*32 + 0..31}) -> HBM ----
     // Store phase: each thread owns one 16-byte chunk column (cc) and, per slab, the IT buffer rows
     // tid / 32 + 8 * it.  What the rows need from HBM (scatter indices, the saved pre-activation of the
-    // SwiGLU backward) is requested in batches before it is used: the indices of all four slabs before the
-    // accumulators are packed, a slab's pre-activations before its first row is processed.
+    // activation backward) is requested in batches before it is used: the indices of all four slabs before the
+    // accumulators are packed (and waited for after that), a slab's pre-activations one slab ahead.
     T* C = reinterpret_cast<T*>(P.c);
     constexpr int C_CHUNKS = BN / PV;             // 32
     constexpr int ROW_STEP = THREADS / C_CHUNKS;  // 8
