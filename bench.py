@@ -179,6 +179,7 @@ def _other_config(workload: dict, steps: int, warmup: int) -> dict:
 
     import flash_model_architectures_amd as xma
     from flash_model_architectures_amd import _native
+    from flash_model_architectures_amd.utils import skewed_router_bias
 
     dev, dt = torch.device("cuda:0"), torch.bfloat16
     T, H, I = workload["tokens"], workload["hidden"], workload["intermediate"]
@@ -192,14 +193,7 @@ def _other_config(workload: dict, steps: int, warmup: int) -> dict:
     if "bias" in workload["routing"]:
         with torch.no_grad():
             raw = moe.gate(x)
-        zipf = -1.2 * torch.log(torch.arange(E, dtype=torch.float32, device=dev) + 1.0)
-        c = 1.0
-        while True:
-            _, selected = xma.topk_softmax(raw + (c * zipf).to(dt), k)
-            if E - int(torch.unique(selected).numel()) >= 4 or c >= 16.0:
-                break
-            c += 0.5
-        bias = (c * zipf).to(dt)
+        bias, c = skewed_router_bias(raw, k)
         moe.gate.register_forward_hook(lambda mod, inp, out: out + bias)
         result["zipf_bias_scale_c"] = c
 

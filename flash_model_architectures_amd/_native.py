@@ -19,6 +19,8 @@ _lib: ctypes.CDLL | None = None
 
 DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
+ABI_VERSION = 3  # XMA_ABI_VERSION of include/xma_hip.h these bindings were written against
+
 GEMM_TN, GEMM_NN, GEMM_MT = 0, 1, 2
 EPI_NONE, EPI_SWIGLU, EPI_SWIGLU_BWD, EPI_GLU, EPI_GLU_BWD, EPI_GELU_TANH, EPI_GELU_TANH_BWD = 0, 1, 2, 3, 4, 5, 6
 
@@ -27,10 +29,12 @@ class GroupedGemmArgs(ctypes.Structure):
     """struct xma_grouped_gemm_args"""
 
     _fields_ = [
+        ("struct_size", ctypes.c_uint32),
         ("kind", c_int32),
         ("dtype", c_int32),
         ("epilogue", c_int32),
         ("num_experts", c_int32),
+        ("reserved", c_int32),
         ("rows", c_int64),
         ("n", c_int64),
         ("k", c_int64),
@@ -61,6 +65,7 @@ PROTOTYPES: dict[str, tuple] = {
     "xma_last_error": (c_char_p, []),
     "xma_version": (c_char_p, []),
     "xma_target_arch": (c_char_p, []),
+    "xma_abi_version": (c_int, []),
     "xma_continuous_count": (c_int, [c_void_p, c_int, c_int64, c_int32, c_void_p, c_void_p]),
     "xma_route_workspace_bytes": (c_int64, [c_int64, c_int32]),
     "xma_route_build": (
@@ -164,6 +169,11 @@ def load() -> ctypes.CDLL:
                 "`python -m flash_model_architectures_amd.build` (needs hipcc); there is no fallback path"
             )
         lib = ctypes.CDLL(_LIB_PATH)
+        if not hasattr(lib, "xma_abi_version") or lib.xma_abi_version() != ABI_VERSION:
+            raise RuntimeError(
+                f"{_LIB_PATH} was built from another revision of include/xma_hip.h than these bindings "
+                f"(ABI version {ABI_VERSION} expected): rebuild it with `python -m flash_model_architectures_amd.build`"
+            )
         for name, (restype, argtypes) in PROTOTYPES.items():
             fn = getattr(lib, name)
             fn.restype = restype

@@ -54,8 +54,20 @@ def _run(cmd: list[str]) -> None:
         print(out, file=sys.stderr)
 
 
-def build(verbose: bool = False, jobs: int | None = None) -> str:
-    """Compile every source in csrc/ and link lib/libxma_hip.so; returns the library path."""
+def _up_to_date(src: str, obj: str) -> bool:
+    """True if `obj` is newer than the source, every header in csrc/ and the public header."""
+
+    if not os.path.exists(obj):
+        return False
+    deps = [os.path.join(CSRC_DIR, src)]
+    deps += [os.path.join(CSRC_DIR, f) for f in os.listdir(CSRC_DIR) if f.endswith(".h")]
+    deps.append(os.path.join(os.path.dirname(_PACKAGE_DIR), "include", "xma_hip.h"))
+    return all(os.path.getmtime(d) <= os.path.getmtime(obj) for d in deps if os.path.exists(d))
+
+
+def build(verbose: bool = False, jobs: int | None = None, incremental: bool = False) -> str:
+    """Compile every source in csrc/ and link lib/libxma_hip.so; returns the library path.  `incremental` (the
+    command line's -i) skips sources whose object file is newer than everything it is built from."""
 
     hipcc = _hipcc()
     os.makedirs(LIB_DIR, exist_ok=True)
@@ -64,6 +76,8 @@ def build(verbose: bool = False, jobs: int | None = None) -> str:
 
     def compile_one(src: str) -> str:
         obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+        if incremental and _up_to_date(src, obj):
+            return obj
         cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC_DIR, src), "-o", obj]
         if verbose:
             print(" ".join(cmd))
@@ -81,4 +95,4 @@ def build(verbose: bool = False, jobs: int | None = None) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv))
+    print(build(verbose="-v" in sys.argv, incremental="-i" in sys.argv))

@@ -31,5 +31,6 @@ extern "C" {
 const char* xma_last_error(void) { return xma::g_error; }
 const char* xma_version(void) { return "0.1.0"; }
 const char* xma_target_arch(void) { return "gfx950"; }
+int xma_abi_version(void) { return XMA_ABI_VERSION; }
 
 }  // extern "C"

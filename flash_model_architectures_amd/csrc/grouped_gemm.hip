@@ -17,6 +17,9 @@
 // tiles (expert, first row), so ragged and empty groups cost nothing; the main kernel renumbers
 // work-groups so that each of the 8 XCDs (private L2 each) owns a contiguous range of tiles, and
 // walks tiles in bands of 4 row tiles x all column tiles to reuse both panels from L2.
+#include <cstddef>
+#include <cstring>
+
 #include "grouped_gemm_common.h"
 
 namespace xma {
@@ -595,7 +598,17 @@ int64_t xma_grouped_gemm_workspace_bytes(int32_t num_experts, int64_t rows) {
 
 int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
     XMA_REQUIRE(args != nullptr, "xma_grouped_gemm: null args");
-    const xma_grouped_gemm_args& a = *args;
+    // The caller says how long its revision of the struct is; fields it does not know are zero / NULL.
+    XMA_REQUIRE(args->struct_size >= offsetof(xma_grouped_gemm_args, workspace_bytes) + sizeof(int64_t) &&
+                    args->struct_size <= sizeof(xma_grouped_gemm_args),
+                "xma_grouped_gemm: struct_size=%u is not a revision of xma_grouped_gemm_args this library knows "
+                "(%zu bytes at ABI version %d)",
+                args->struct_size, sizeof(xma_grouped_gemm_args), XMA_ABI_VERSION);
+    xma_grouped_gemm_args copy;
+    memset(&copy, 0, sizeof(copy));
+    memcpy(&copy, args, args->struct_size);
+    const xma_grouped_gemm_args& a = copy;
+    XMA_REQUIRE(a.reserved == 0, "xma_grouped_gemm: reserved field must be 0");
     XMA_REQUIRE(valid_dtype(a.dtype), "xma_grouped_gemm: bad dtype %d", a.dtype);
     XMA_REQUIRE(a.kind >= XMA_GEMM_TN && a.kind <= XMA_GEMM_MT, "xma_grouped_gemm: bad kind %d", a.kind);
     XMA_REQUIRE(a.num_experts >= 1 && a.num_experts <= 16384, "xma_grouped_gemm: num_experts=%d outside [1, 16384]",

@@ -63,16 +63,35 @@ def exclusive_offsets(expert_offsets: torch.Tensor, E: int) -> torch.Tensor:
 
 # One workspace per (device, stream), grown on demand and reused by every launch on that stream: launches on a
 # stream run in order, and every kernel initialises the part of the workspace it reads.
+#
+# Lifetime and sharing rules:
+#   * a buffer lives until release_workspaces() or the end of the process; a stream that has run a 16-bit grouped GEMM
+#     holds at least the 64 MiB split-K region;
+#   * ONE user at a time: the buffer serves, in turn, as tile tables and split-K region of a grouped GEMM, as the
+#     per-chunk histograms of route_build and as the inverted index of `ungroup`.  An operator must never need two of
+#     these in one launch, and must not expect the contents to survive the next operator on the stream;
+#   * under stream capture (CUDA graphs) nothing is cached: a buffer allocated during capture belongs to the graph's
+#     private pool and must not be handed to later eager launches, so every captured call gets a buffer of its own
+#     (kept alive by the graph's pool for its replays).
 _workspaces: dict[tuple[int, int], torch.Tensor] = {}
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
     key = (device.index if device.index is not None else torch.cuda.current_device(), nat.stream())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def release_workspaces() -> None:
+    """Drop every cached workspace (they are re-created on demand).  The caller must make sure no launch that uses
+    one is still running, e.g. by synchronising the streams first."""
+
+    _workspaces.clear()
 
 
 def offsets_from_sorted(sorted_expert_idxs: torch.Tensor, E: int) -> torch.Tensor:
@@ -494,6 +513,7 @@ def _grouped_gemm(
         assert in_index.dtype == out_index.dtype
     index = in_index if in_index is not None else out_index
     args = nat.GroupedGemmArgs()
+    args.struct_size = ctypes.sizeof(nat.GroupedGemmArgs)
     args.kind, args.dtype, args.epilogue, args.num_experts = kind, nat.dtype_code(a), epilogue, E
     args.rows, args.n, args.k = rows, n, k
     args.a, args.lda = a.data_ptr(), lda

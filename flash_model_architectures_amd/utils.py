@@ -38,3 +38,29 @@ def empty_like_contiguous(x: torch.Tensor, dtype: torch.dtype | None = None) -> 
 class XMAModule(nn.Module):
     def extra_repr(self) -> str:
         return f"# parameters = {sum(p.numel() for p in self.parameters()):,}"
+
+
+def zipf_router_bias(num_experts: int, s: float = 1.2, device=None) -> torch.Tensor:
+    """fp32[num_experts], `-s * ln(e + 1)`: a Zipf(s) prior over the expert index in log space.  Added to the router
+    logits (times a scale c) it overloads the first experts and starves the last ones."""
+
+    return -s * torch.log(torch.arange(num_experts, dtype=torch.float32, device=device) + 1.0)
+
+
+def skewed_router_bias(raw_logits: torch.Tensor, top_k: int, s: float = 1.2, min_empty: int = 4,
+                       c_start: float = 1.0, c_step: float = 0.5, c_max: float = 16.0) -> tuple[torch.Tensor, float]:
+    """Bias of the skewed-routing workload for a layer whose unbiased router logits are `raw_logits` [T, E]:
+    `c * zipf_router_bias(E, s)` in the logits' dtype, with c raised from `c_start` in steps of `c_step` until at
+    least `min_empty` experts receive no token under top-k selection (or c reaches `c_max`).  Returns (bias, c).
+    The benchmark and the parity test of that workload both call this, so they run the same routing."""
+
+    from .functional import topk_softmax
+
+    zipf = zipf_router_bias(raw_logits.size(-1), s, raw_logits.device)
+    c = c_start
+    while True:
+        bias = (c * zipf).to(raw_logits.dtype)
+        _, selected = topk_softmax(raw_logits + bias, top_k)
+        if raw_logits.size(-1) - int(torch.unique(selected).numel()) >= min_empty or c >= c_max:
+            return bias, c
+        c += c_step

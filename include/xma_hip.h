@@ -64,11 +64,19 @@ enum xma_gemm_epilogue {
     XMA_EPI_GELU_TANH_BWD = 6
 };
 
+/* ABI revision of this header: bumped whenever a struct gains a field or an enum a value.  A caller may compare it
+   with xma_abi_version() of the library it loaded. */
+#define XMA_ABI_VERSION 3
+
 typedef struct xma_grouped_gemm_args {
+    uint32_t struct_size; /* sizeof(xma_grouped_gemm_args) as the CALLER was compiled: fields beyond it are taken as
+                             zero / NULL, so a caller built against a shorter revision of the struct keeps working;
+                             0 or a size larger than the library's is rejected */
     int32_t kind;      /* enum xma_gemm_kind */
     int32_t dtype;     /* enum xma_dtype of A, B, C, aux */
     int32_t epilogue;  /* enum xma_gemm_epilogue */
     int32_t num_experts;
+    int32_t reserved;  /* 0 */
     int64_t rows;      /* routed rows M = T * top_k (the ragged dimension) */
     int64_t n;         /* TN/NN: output columns.  MT: columns of A (rows of each C[e]) */
     int64_t k;         /* TN/NN: reduction length.  MT: columns of B (columns of each C[e]) */
@@ -106,6 +114,8 @@ const char* xma_last_error(void);
 /* Library version and the GPU architecture the code objects were built for ("gfx950"). */
 const char* xma_version(void);
 const char* xma_target_arch(void);
+/* XMA_ABI_VERSION of the header the library was built from. */
+int xma_abi_version(void);
 
 /*
  * Histogram of ids in [0, bins) into counts[bins] (uint32).  ids: int32 or int64, n < 2^32.

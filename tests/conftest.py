@@ -35,15 +35,15 @@ def pytest_terminal_summary(terminalreporter):
     from tests import helpers
 
     by_tol: dict = {}
-    for what, tol, err, elem, floor in helpers.WORST:
-        cur = by_tol.setdefault((tol, floor), [0.0, "", 0.0, ""])
+    for what, tol, err, elem, floor, elem_tol in helpers.WORST:
+        cur = by_tol.setdefault((tol, floor, elem_tol), [0.0, "", 0.0, ""])
         if err > cur[0]:
             cur[0], cur[1] = err, what
         if elem > cur[2]:
             cur[2], cur[3] = elem, what
-    for tol, floor in sorted(by_tol):
-        err, what_err, elem, what_elem = by_tol[(tol, floor)]
+    for tol, floor, elem_tol in sorted(by_tol):
+        err, what_err, elem, what_elem = by_tol[(tol, floor, elem_tol)]
         terminalreporter.write_line(
             f"parity, bar {tol:.0e}: worst whole-tensor error {err:.2e} ({what_err}), worst element-wise error "
-            f"|a-b| / (|b| + {floor:g} rms) {elem:.2e} ({what_elem}) against {2 * tol:.0e}"
+            f"|a-b| / (|b| + {floor:g} rms) {elem:.2e} ({what_elem}) against {elem_tol:.1e}"
         )

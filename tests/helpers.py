@@ -7,19 +7,34 @@ import math
 import torch
 
 
-# Tolerances of the parity bar.  TOL bounds the whole tensor: max |a - b| / max |b| <= TOL.  On top of that every
-# element is held to its own scale: |a - b| <= ELEM_TOL * (|b| + F * rms(b)), so that an element far below the tensor's
-# largest cannot hide a large relative error behind it.  The rms term is the floor that the rounding of the 16-bit
-# intermediates sets for an element whose terms cancel; for a stack of per-expert matrices it is taken per expert.
-# ELEM_TOL is twice TOL: relative to the rms, rather than to the largest element, the roundings of the (up to five)
-# intermediates of a backward pass show in full (measured on the layer tests: up to 1.1 x TOL for outputs and input
-# gradients).  F is 1 except for weight gradients that sum only a handful of rows per expert (the reference's
-# seven-token shapes, full-size layers with a sampled upstream gradient, experts that Zipf routing leaves almost
-# empty): there the products of two heavy-tailed factors are not averaged, single terms reach many times the rms,
-# and so does their rounding; those calls pass F = FEW_ROWS_FLOOR (measured need: up to 4).
+# Tolerances of the parity bar.
+#
+# TOL is the workload definition's figure per dtype ("max relative error <= 1e-5 in fp32, <= 2e-2 in bf16 with fp32
+# accumulation"; fp16, which the definition does not name, is held to 5e-3) and bounds the whole tensor:
+# max |a - b| / max |b| <= TOL.
+#
+# On top of that every element is held to its own scale, |a - b| <= E * (|b| + F * rms(b)), so that an element far
+# below the tensor's largest cannot hide a large relative error behind it.  The rms term is the floor that rounding
+# sets for an element whose terms cancel; for a stack of per-expert matrices it is taken per expert.  E depends on
+# what the checker computes:
+#   * GEMM_ELEM_TOL: one GEMM against fp32 matmuls over the SAME 16-bit-valued operands.  The only differences are
+#     the summation order and the final rounding of the output, at most half a unit in the last place: 2^-8 of the
+#     value for bf16 (8 significant bits), 2^-11 for fp16.  The bar is that half unit plus 1e-4 for the summation
+#     order; 1e-5 for fp32.  Measured on 2048-row reductions: 3.1e-3 (bf16).
+#   * ELEM_TOL (the default of assert_close): a whole layer against the oracle evaluated without intermediate
+#     rounding (in fp32 for the 16-bit types, in float64 for fp32 layers), while the kernel path (like the
+#     reference's) stores up to five intermediates per gradient in the layer's type (pre-activation, activation,
+#     weighted upstream gradient, activation gradient, result).  Relative to the rms, rather than to the largest
+#     element, these roundings show in full: measured up to 1.6 x TOL for bf16, 0.8 x TOL for fp16, 1.1 x TOL for fp32
+#     (reductions of 8192 terms accumulated in fp32, against float64).  The bar is 2 x TOL.
+# F is 1 except for weight gradients that sum only a handful of rows per expert (the reference's seven-token
+# shapes, full-size layers with a sampled upstream gradient, experts that Zipf routing leaves almost empty): there
+# the products of two heavy-tailed factors are not averaged, single terms reach many times the rms, and so does their
+# rounding; those calls pass F = FEW_ROWS_FLOOR (measured: 3.97e-2 at F = 4, which sits on the bar, 2.2e-2 at F = 8).
 TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 5e-3}
-ELEM_TOL = {tol: 2.0 * tol for tol in (1e-5, 2e-2, 5e-3)}
-FEW_ROWS_FLOOR = 8.0
+ELEM_TOL = {1e-5: 2e-5, 2e-2: 4e-2, 5e-3: 1e-2}
+GEMM_ELEM_TOL = {torch.float32: 1e-5, torch.bfloat16: 2.0**-8 + 1e-4, torch.float16: 2.0**-11 + 1e-4}
+FEW_ROWS_FLOOR = 6.0
 
 # absolute tolerances (rtol 0) of the reference's own MoE test for output, dX and dW
 # (tests/layers/moe_test.py:112-122, :130-140, :146-156)
@@ -69,15 +84,17 @@ def max_elementwise_err(got: torch.Tensor, want: torch.Tensor, floor: float = 1.
     return worst
 
 
-def assert_close(got: torch.Tensor, want: torch.Tensor, tol: float, what: str = "", floor: float = 1.0) -> None:
-    """Both parity checks: the whole tensor against `tol`, every element against twice that on its own scale (see
-    TOL / ELEM_TOL; `floor` is the F described there)."""
+def assert_close(got: torch.Tensor, want: torch.Tensor, tol: float, what: str = "", floor: float = 1.0,
+                 elem_tol: float | None = None) -> None:
+    """Both parity checks: the whole tensor against `tol`, every element on its own scale against `elem_tol`
+    (default: ELEM_TOL of `tol`; `floor` is the F described there)."""
 
     err = max_rel_err(got, want)
     assert math.isfinite(err) and err <= tol, f"{what}: max relative error {err:.3e} > {tol:.1e}"
     elem = max_elementwise_err(got, want, floor)
-    elem_tol = ELEM_TOL.get(tol, 2.0 * tol)
-    WORST.append((what, tol, err, elem, floor))
+    if elem_tol is None:
+        elem_tol = ELEM_TOL.get(tol, 2.0 * tol)
+    WORST.append((what, tol, err, elem, floor, elem_tol))
     assert math.isfinite(elem) and elem <= elem_tol, (
         f"{what}: worst element |a-b| / (|b| + {floor:g} rms(b)) = {elem:.3e} > {elem_tol:.1e}"
     )

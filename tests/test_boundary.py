@@ -129,3 +129,35 @@ def test_experts_methods_with_the_reference_names(add_bias):
     again = down_d.torch_forward(parts, None, return_list=False)
     want_again = to.experts_forward(want_h, down.weight, r.expert_frequency, False, down.bias)
     assert_close(again, want_again.detach(), 1e-5, "torch_forward on a list")
+
+
+def test_shorter_revision_of_the_gemm_argument_struct():
+    """A caller compiled against the revision of xma_grouped_gemm_args that ended with `workspace_bytes` passes that
+    size in `struct_size`; whatever follows its struct in memory must not be read as the bias pointer."""
+
+    import ctypes
+
+    from flash_model_architectures_amd import _native as nat
+
+    dev = "cuda"
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(64, 64, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(2, 32, 64, generator=g) * 0.1).to(torch.bfloat16).to(dev)
+    off = torch.tensor([0, 40, 64], dtype=torch.int32, device=dev)
+    out = torch.empty(64, 32, dtype=torch.bfloat16, device=dev)
+    lib = nat.load()
+    ws = torch.empty(lib.xma_grouped_gemm_workspace_bytes(2, 64), dtype=torch.uint8, device=dev)
+    args = nat.GroupedGemmArgs()
+    args.struct_size = nat.GroupedGemmArgs.bias.offset  # the older, shorter struct
+    args.kind, args.dtype, args.epilogue, args.num_experts = nat.GEMM_TN, nat.DTYPE_CODE[torch.bfloat16], nat.EPI_NONE, 2
+    args.rows, args.n, args.k = 64, 32, 64
+    args.a, args.lda = x.data_ptr(), 64
+    args.b, args.ldb, args.b_expert_stride = w.data_ptr(), 64, 32 * 64
+    args.c, args.ldc = out.data_ptr(), 32
+    args.expert_offsets = off.data_ptr()
+    args.in_fan_out = 1
+    args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
+    args.bias, args.ld_bias = 0xDEAD0000, 12345  # memory past the caller's struct: must be ignored
+    nat.call("xma_grouped_gemm", ctypes.byref(args), nat.stream())
+    ref = torch.cat([x[:40].float() @ w[0].float().T, x[40:].float() @ w[1].float().T])
+    assert_close(out, ref, 2e-2)

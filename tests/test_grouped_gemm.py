@@ -8,7 +8,7 @@ import torch
 from flash_model_architectures_amd import ops
 from oracle import torch_oracle as to
 
-from .helpers import TOL, assert_close
+from .helpers import GEMM_ELEM_TOL, TOL, assert_close
 
 pytestmark = pytest.mark.gpu
 
@@ -181,6 +181,65 @@ def test_fused_activations_and_bias(case, activation, dtype):
     assert_close(d_pre, leaf.grad, tol, f"fused {activation} backward")
 
 
+def test_full_length_reductions_dense():
+    """Every layout once at the row counts of the benchmark layer (16384 routed rows over 8 experts, about 2048 per
+    expert) with DENSE operands, so that the weight-gradient kernel's reductions run over ~2048 non-zero rows (32
+    stages) and every output element is a full-length sum.  Checker: per-expert fp32 matmuls on the device over the
+    same 16-bit-valued operands (a library routine), so the only differences are the summation order and the one
+    final rounding; every element is held to the single-GEMM bar (GEMM_ELEM_TOL, F = 1)."""
+
+    dtype, dev = torch.bfloat16, "cuda"
+    T, H, I, E, k = 8192, 1024, 512, 8, 2
+    M = T * k
+    tol = TOL[dtype]
+    g = torch.Generator().manual_seed(2024)
+    x = torch.randn(T, H, generator=g).to(dtype).to(dev)
+    w1 = (torch.randn(E, 2 * I, H, generator=g) * 0.05).to(dtype).to(dev)
+    w2 = (torch.randn(E, H, I, generator=g) * 0.05).to(dtype).to(dev)
+    d_pre = torch.randn(M, 2 * I, generator=g).to(dtype).to(dev)
+    dyg = torch.randn(M, H, generator=g).to(dtype).to(dev)
+    act = torch.randn(M, I, generator=g).to(dtype).to(dev)
+    r = _routing(T, E, k, 77)
+    off = r.expert_offsets.tolist()
+    assert min(off[e + 1] - off[e] for e in range(E)) > 1536
+    idxd, offd, sed = r.sorted_scattered_idxs.to(dev).int(), r.expert_offsets.to(dev), r.sorted_expert_idxs.to(dev).int()
+    xg = x[(idxd // k).long()].float()
+
+    def per_expert(fn):
+        return torch.cat([fn(e, slice(off[e], off[e + 1])) for e in range(E)])
+
+    def stacked(fn):
+        return torch.stack([fn(e, slice(off[e], off[e + 1])) for e in range(E)])
+
+    elem = GEMM_ELEM_TOL[dtype]
+    h = torch.empty(M, 2 * I, dtype=dtype, device=dev)
+    ops.scatter2scatter(x, w1.permute(0, 2, 1), sed, idxd, h, k, False, True, offd)
+    assert_close(h, per_expert(lambda e, s: xg[s] @ w1[e].float().T), tol, "dense: up projection (TN)", elem_tol=elem)
+
+    d_act = torch.empty(M, I, dtype=dtype, device=dev)
+    ops.scatter2scatter(dyg, w2, sed, idxd, d_act, 1, True, True, offd)
+    assert_close(d_act, per_expert(lambda e, s: dyg[s].float() @ w2[e].float()), tol, "dense: input gradient (NN)", elem_tol=elem)
+
+    d_xe = torch.empty(M, H, dtype=dtype, device=dev)
+    ops.scatter2scatter(d_pre, w1, sed, idxd, d_xe, 1, True, False, offd)
+    ref = torch.empty(M, H, device=dev)
+    ref[idxd.long()] = per_expert(lambda e, s: d_pre[s].float() @ w1[e].float())
+    assert_close(d_xe, ref, tol, "dense: scattered input gradient (NN)", elem_tol=elem)
+
+    # weight gradients: reductions over every row of the expert, with and without the fused token gather
+    d_w1 = torch.full((E, 2 * I, H), float("nan"), dtype=dtype, device=dev)
+    ops.group_bwd_W(d_pre, x, offd, d_w1.permute(0, 2, 1), E, idxd, k)
+    want = stacked(lambda e, s: d_pre[s].float().T @ xg[s])
+    assert_close(d_w1, want, tol, "dense: up weight gradient (MT, fused gather)", elem_tol=elem)
+    xg16 = x[(idxd // k).long()]
+    d_w1b = torch.full((E, 2 * I, H), float("nan"), dtype=dtype, device=dev)
+    ops.group_bwd_W(d_pre, xg16, offd, d_w1b.permute(0, 2, 1), E)
+    assert_close(d_w1b, want, tol, "dense: up weight gradient (MT)", elem_tol=elem)
+    d_w2 = torch.full((E, H, I), float("nan"), dtype=dtype, device=dev)
+    ops.group_bwd_W(dyg, act, offd, d_w2.permute(0, 2, 1), E)
+    assert_close(d_w2, stacked(lambda e, s: dyg[s].float().T @ act[s].float()), tol, "dense: down weight gradient (MT)", elem_tol=elem)
+
+
 def test_argument_validation():
     dev = "cuda"
     x = torch.randn(8, 64, device=dev, dtype=torch.bfloat16)
@@ -257,6 +316,79 @@ def test_whole_rounds_plus_split_remainder(layout, K):
         assert_close(outs[0], ref, TOL[torch.bfloat16])
         for out in outs[1:]:
             assert torch.equal(outs[0], out)
+
+
+@pytest.mark.parametrize("K", [4160, 6200, 8320])
+@pytest.mark.parametrize("form", ["TN", "TN+swiglu", "NN", "NN+swiglu_bwd"])
+def test_split_remainder_exact_sums(form, K):
+    """The split of a partly filled last round (reductions cut in 2, 3 and 4 parts at these K) on all four
+    row-grouped instantiations, with operands made of small integers: every product and every partial sum is then
+    exact in fp32 whatever the order, so the stored product must equal the correctly rounded exact matmul BIT FOR
+    BIT.  A partial sum that is lost, counted twice, or picked up from an earlier launch (the exchange memory is
+    reused: two operand sets alternate) changes an integer and fails the comparison.  The fused activations are
+    checked on top of the exact product: the stored pre-activation bit for bit, the activation values within the
+    bar."""
+
+    dev, dt = "cuda", torch.bfloat16
+    E, N = 4, 1792  # 7 column tiles of the output; ~43 row tiles -> ~300 tiles on 256 compute units
+    sizes = [2700, 1, 3100, 4300]
+    M = sum(sizes)
+    g = torch.Generator().manual_seed(17 + K)
+    off_list = [0] + torch.tensor(sizes).cumsum(0).tolist()
+    off = torch.tensor(off_list, dtype=torch.int32, device=dev)
+    idx = torch.arange(M, dtype=torch.int32, device=dev)
+    se = torch.repeat_interleave(torch.arange(E), torch.tensor(sizes)).int().to(dev)
+    gated = form == "TN+swiglu"
+    n_w = 2 * N if gated else N
+
+    def exact(a, w):  # [M, n_w] fp32, exact: integer operands, |sums| < 2^24
+        return torch.cat([a[off_list[e] : off_list[e + 1]].float() @ w[e].float().T for e in range(E)])
+
+    sets = []
+    for _ in range(2):
+        a = torch.randint(-2, 3, (M, K), generator=g).to(dt).to(dev)
+        w = torch.randint(-1, 2, (E, n_w, K), generator=g).to(dt).to(dev)  # [E, N, K]
+        sets.append((a, w, exact(a, w)))
+    pre_in = (torch.randn(M, 2 * N, generator=g)).to(dt).to(dev)  # saved pre-activation of the backward form
+
+    def run(a, w):
+        if form == "TN":
+            out = torch.empty(M, N, dtype=dt, device=dev)
+            ops.scatter2scatter(a, w.permute(0, 2, 1), se, idx, out, 1, True, True, off)
+            return (out,)
+        if form == "TN+swiglu":
+            act = torch.empty(M, N, dtype=dt, device=dev)
+            pre = torch.empty(M, 2 * N, dtype=dt, device=dev)
+            ops.up_projection_fused(a, w, idx, off, act, pre, 1, "swiglu")
+            return pre, act
+        w_kn = w.permute(0, 2, 1).contiguous()  # [E, K, N], N contiguous
+        if form == "NN":
+            out = torch.empty(M, N, dtype=dt, device=dev)
+            ops.scatter2scatter(a, w_kn, se, idx, out, 1, True, True, off)
+            return (out,)
+        d_pre = torch.empty(M, 2 * N, dtype=dt, device=dev)
+        ops.down_projection_dgrad_fused(a, w_kn, pre_in, off, d_pre, "swiglu")
+        return (d_pre,)
+
+    results = [[], []]
+    for _ in range(3):
+        for i, (a, w, _) in enumerate(sets):
+            results[i].append(run(a, w))
+    for i, (a, w, want) in enumerate(sets):
+        first = results[i][0]
+        for later in results[i][1:]:
+            for x, y in zip(first, later):
+                assert torch.equal(x, y), "results of one operand set differ between launches"
+        if form in ("TN", "NN"):
+            assert torch.equal(first[0], want.to(dt)), "product differs from the correctly rounded exact sums"
+        elif form == "TN+swiglu":
+            pre, act = first
+            assert torch.equal(pre, want.to(dt)), "pre-activation differs from the correctly rounded exact sums"
+            assert_close(act, to.swiglu_packed(pre.cpu()), TOL[dt], "activation of a split tile")
+        else:
+            pc = pre_in.cpu()
+            dg, du = to.swiglu_backward(pc[:, N:], pc[:, :N], want.cpu())
+            assert_close(first[0], torch.cat([du, dg], -1), TOL[dt], "activation backward of a split tile")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])

@@ -19,6 +19,8 @@ import torch.nn.functional as F
 import flash_model_architectures_amd as xma
 from oracle import torch_oracle as to
 
+from flash_model_architectures_amd.utils import skewed_router_bias
+
 from .helpers import FEW_ROWS_FLOOR, REFERENCE_ATOL, TOL, assert_close, assert_same_ints, make_moe_inputs, zipf_bias
 
 pytestmark = pytest.mark.gpu
@@ -67,20 +69,22 @@ def _run_case(T, H, I, E, k, dtype, activation="swiglu", seed=0, bias=None, back
     assert_same_ints(selected, want_selected, "selected experts")
 
     # value parity: oracle in fp32 on the same (dtype-valued) inputs and the same selection
-    od = oracle_dtype or torch.float32
+    # fp32 layers: the oracle runs in float64, so that the comparison sees the kernels' error alone
+    od = oracle_dtype or (torch.float64 if dtype == torch.float32 else torch.float32)
+    elem = None
     xo, go, uo, do = (t.to(od).clone().requires_grad_() for t in (x, w_gate, w_up, w_down))
     yo, logits_o = _oracle_on_selection(xo, go, uo, do, want_selected, act_cpu, None if bias is None else bias.to(od))
     tol = TOL[dtype]
-    assert_close(logits, logits_o, tol, "router logits")
-    assert_close(y, yo, tol, "output")
+    assert_close(logits, logits_o, tol, "router logits", elem_tol=elem)
+    assert_close(y, yo, tol, "output", elem_tol=elem)
     if not backward:
         return
     y.backward(d_y.cuda())
     yo.backward(d_y.to(od))
-    assert_close(xd.grad, xo.grad, tol, "dX")
+    assert_close(xd.grad, xo.grad, tol, "dX", elem_tol=elem)
     floor = FEW_ROWS_FLOOR if few_rows else 1.0  # weight gradients that sum only a handful of rows per expert
-    assert_close(moe.c_fc.weight.grad, uo.grad, tol, "dW up", floor)
-    assert_close(moe.c_proj.weight.grad, do.grad, tol, "dW down", floor)
+    assert_close(moe.c_fc.weight.grad, uo.grad, tol, "dW up", floor, elem_tol=elem)
+    assert_close(moe.c_proj.weight.grad, do.grad, tol, "dW down", floor, elem_tol=elem)
     assert_close(moe.gate.weight.grad, go.grad, 5 * tol, "dW gate", floor)
     if not reference_atol:
         return
@@ -207,25 +211,26 @@ def test_fused_and_general_pipelines_agree():
     assert torch.equal(fused.c_proj.weight.grad, general.c_proj.weight.grad)
 
 
-def _full_size_sampled(T, H, I, E, k, sample, bias=None):
+def _full_size_sampled(T, H, I, E, k, sample, skewed=False):
     """A whole bf16 layer, forward and backward, at its real shape on the GPU, checked against the oracle on a
     sample of tokens.  Every token's output depends on that token alone, and with an upstream gradient that is
     zero outside the sample every gradient depends on the sample alone, so the oracle only has to evaluate the
-    sample while the kernels run the whole layer.  Returns the expert histogram."""
+    sample while the kernels run the whole layer.  `sample` is a list of tokens or a function of the selected
+    experts [T, k] and the expert histogram that returns one (so that a test can aim at particular experts).
+    `skewed`: the router bias of the skewed-routing workload, built exactly as the benchmark builds it.
+    Returns the expert histogram and the layer (with its gradients)."""
 
     dt, dev = torch.bfloat16, "cuda"
     torch.manual_seed(0)
     moe = xma.MoE(E, k, H, I, xma.swiglu_packed, True, False, 0.02).to(dt).to(dev)
-    if bias is not None:
-        moe.gate.register_forward_hook(lambda mod, inp, out: out + bias.to(out))
     x = torch.randn(T, H, device=dev).to(dt).requires_grad_()
-    sample = torch.as_tensor(sample)
-    on_dev = sample.to(dev)
-    d_y = torch.zeros(T, H, device=dev, dtype=dt)
-    d_y[on_dev] = torch.randn(len(sample), H, device=dev).to(dt)
+    bias = None
+    if skewed:
+        with torch.no_grad():
+            bias, _ = skewed_router_bias(moe.gate(x), k)
+        moe.gate.register_forward_hook(lambda mod, inp, out: out + bias)
 
     y, logits = moe(x)
-    y.backward(d_y)
 
     # routing integers on the GPU's own logits: selection, histogram, offsets and permutation bit-exact
     _, selected = xma.topk_softmax(logits.detach(), k)
@@ -240,12 +245,20 @@ def _full_size_sampled(T, H, I, E, k, sample, bias=None):
     counts = want_routing.expert_frequency.to(torch.int64)
     assert int(counts.sum()) == T * k
 
+    if callable(sample):
+        sample = sample(want_selected, counts)
+    sample = torch.as_tensor(sorted(set(int(t) for t in sample)))
+    on_dev = sample.to(dev)
+    d_y = torch.zeros(T, H, device=dev, dtype=dt)
+    d_y[on_dev] = torch.randn(len(sample), H, device=dev).to(dt)
+    y.backward(d_y)
+
     xs = x.detach()[on_dev].cpu().float().requires_grad_()
     w_gate = moe.gate.weight.detach().cpu().float()
     w_up = moe.c_fc.weight.detach().cpu().float().requires_grad_()
     w_down = moe.c_proj.weight.detach().cpu().float().requires_grad_()
     ys, _ = _oracle_on_selection(xs, w_gate, w_up, w_down, want_selected[sample], to.swiglu_packed,
-                                 None if bias is None else bias.float())
+                                 None if bias is None else bias.cpu().float())
     ys.backward(d_y[on_dev].cpu().float())
 
     tol = TOL[dt]
@@ -259,13 +272,13 @@ def _full_size_sampled(T, H, I, E, k, sample, bias=None):
     assert_close(moe.c_fc.weight.grad, w_up.grad, tol, "dW up", FEW_ROWS_FLOOR)
     assert_close(moe.c_proj.weight.grad, w_down.grad, tol, "dW down", FEW_ROWS_FLOOR)
     assert bool(torch.isfinite(y).all())
-    return counts
+    return counts, moe
 
 
 def test_mixtral_shaped_full_size_sampled():
     """bf16, H 4096, I 14336, 8 experts, top-2, 8192 tokens: near-uniform expert loads from the linear gate."""
 
-    counts = _full_size_sampled(8192, 4096, 14336, 8, 2, [0, 1, 17, 4095, 4096, 6000, 8190, 8191])
+    counts, _ = _full_size_sampled(8192, 4096, 14336, 8, 2, [0, 1, 17, 4095, 4096, 6000, 8190, 8191])
     assert int(counts.min()) > 0
 
 
@@ -273,8 +286,37 @@ def test_fine_grained_full_size_sampled():
     """bf16, H 2048, I 1024, 64 experts, top-6, 16384 tokens (98304 routed rows, about 1536 per expert)."""
 
     sample = [0, 1, 2, 63, 64, 1000, 4095, 4096, 8191, 8192, 12000, 12001, 16000, 16382, 16383, 777]
-    counts = _full_size_sampled(16384, 2048, 1024, 64, 6, sample)
+    counts, _ = _full_size_sampled(16384, 2048, 1024, 64, 6, sample)
     assert int(counts.min()) > 0 and int(counts.max()) < 4 * 1536
+
+
+def test_skewed_routing_full_size_sampled():
+    """bf16, H 2048, I 768, 128 experts, top-8, 16384 tokens (131072 routed rows) with the Zipf(1.2) router bias of
+    the skewed-routing workload, scaled as the benchmark scales it (same seed, same layer, same helper): some experts
+    are overloaded, many are empty.  The sample takes tokens routed to the rarest non-empty experts (one or two rows
+    each: the tail tiles), tokens of the largest expert (first, middle and last of its rows) and a few fixed ones.
+    Asserts bit-exact routing (in the helper), at least four empty experts, one expert far above the mean, and exact
+    zeros in the weight gradients of every empty expert."""
+
+    T, E, k = 16384, 128, 8
+
+    def pick(selected, counts):
+        tokens = [0, 1, 4095, 8192, T - 1]
+        nonempty = [e for e in range(E) if counts[e] > 0]
+        for e in sorted(nonempty, key=lambda e: (int(counts[e]), e))[:6]:  # the rarest experts that have rows
+            rows = (selected == e).any(dim=1).nonzero().flatten().tolist()
+            tokens += [rows[0], rows[-1]]
+        largest = int(counts.argmax())
+        rows = (selected == largest).any(dim=1).nonzero().flatten().tolist()
+        tokens += [rows[0], rows[len(rows) // 2], rows[-1]]
+        return tokens
+
+    counts, moe = _full_size_sampled(T, 2048, 768, E, k, pick, skewed=True)
+    empty = (counts == 0).nonzero().flatten().tolist()
+    assert len(empty) >= 4, f"only {len(empty)} empty experts"
+    assert int(counts.max()) > 4 * T * k // E, "no overloaded expert"
+    for grad in (moe.c_fc.weight.grad, moe.c_proj.weight.grad):
+        assert bool(torch.all(grad[torch.as_tensor(empty, device=grad.device)] == 0)), "empty experts must get zero gradients"
 
 
 def test_backward_of_an_expanded_gradient():

@@ -67,6 +67,10 @@ def test_identification_and_error_channel():
     assert rc != 0 and "k=" in _native.last_error()
     args = _native.GroupedGemmArgs()
     args.kind, args.dtype, args.num_experts = 0, 2, 0
+    assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "struct_size" in _native.last_error()
+    args.struct_size = ctypes.sizeof(args) + 8  # a caller newer than the library
+    assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "struct_size" in _native.last_error()
+    args.struct_size = ctypes.sizeof(args)
     assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "num_experts" in _native.last_error()
     args.num_experts, args.n, args.k = 4, 12, 64  # n not a multiple of 8
     off = (ctypes.c_int32 * 5)()
@@ -81,8 +85,11 @@ def test_struct_layout_matches_header_field_order():
     text = open(HEADER).read()
     body = text[text.index("typedef struct xma_grouped_gemm_args {") : text.index("} xma_grouped_gemm_args;")]
     body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
-    fields = re.findall(r"\b(?:const\s+)?(?:void|int32_t|int64_t)\s*\*?\s*([a-z_0-9]+)\s*;", body)
+    fields = re.findall(r"\b(?:const\s+)?(?:void|uint32_t|int32_t|int64_t)\s*\*?\s*([a-z_0-9]+)\s*;", body)
     assert fields == [f[0] for f in _native.GroupedGemmArgs._fields_]
+    assert fields[0] == "struct_size"
+    version = int(re.search(r"#define XMA_ABI_VERSION (\d+)", text).group(1))
+    assert version == _native.ABI_VERSION == _native.load().xma_abi_version()
 
 
 def test_public_surface_mirrors_the_reference_names():
