@@ -232,23 +232,44 @@ struct OperandLoads {
     }
 
     // Issue this wave's loads I0 <= i < I1 of the stage `stage` into the tile at slab_base + tile_off.
-    template <int I0, int I1>
+    // MASKED = false is for a stage that lies wholly inside the reduction, of a tile none of whose rows and columns
+    // is missing (all_valid): the address is the lane's pointer plus a wave-uniform offset and nothing is compared
+    // or selected.  A wave that is alone on its SIMD pays an issue slot for every instruction, and the masked form
+    // spends five on each load (a 64-bit compare, a mask and, two selects), the plain one none.
+    template <int I0, int I1, bool MASKED>
     __device__ __forceinline__ void issue(char* slab_base, int tile_off, int64_t stage, int64_t red_len) const {
         const int64_t red_left = red_len - stage * BK;  // wave-uniform
         const int64_t stage_off = stage * step;
 #pragma unroll
         for (int i = I0; i < I1; ++i) {
-            const bool ok = valid[PLAN == PLAN_STRIDED ? 0 : i] && (red0 + i * RED_STRIDE < red_left);
             const T* p;
             if constexpr (PLAN == PLAN_ROWS) p = ptr[i] + stage_off;
             else p = ptr[0] + (stage_off + i * load_stride + (i >= LOADS / 2 ? mid_jump : 0));
-            // computed for every lane and then selected: a branch around the load would make the number of
-            // loads in flight differ between waves
-            asm("" : "+v"(p));
-            p = ok ? p : zero_page();
+            if constexpr (MASKED) {
+                const bool ok = valid[PLAN == PLAN_STRIDED ? 0 : i] && (red0 + i * RED_STRIDE < red_left);
+                // computed for every lane and then selected: a branch around the load would make the number of
+                // loads in flight differ between waves
+                asm("" : "+v"(p));
+                p = ok ? p : zero_page();
+            }
+            // The wave's share of the LDS address goes through an empty asm that also names the stage, so that the
+            // address of every load is ONE scalar add on the spot; left alone, the compiler forms all eighty
+            // addresses of a trip round the ring ahead of the loop, runs out of scalar registers and reads them
+            // back from vector lanes.  (Not volatile: a volatile asm fences the instruction scheduler, which
+            // then cannot spread the loads and LDS reads between the matrix instructions.)
+            int w = wave_lds;
+            asm("" : "+s"(w) : "s"((int)stage));
             __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(p),
-                                             XMA_LDS(slab_base + (tile_off + i * NUM_WAVES * 1024 + wave_lds)), 16, 0, 0);
+                                             XMA_LDS(slab_base + (tile_off + i * NUM_WAVES * 1024 + w)), 16, 0, 0);
         }
+    }
+
+    // true when no row or column of this wave's share of the operand tile is missing
+    __device__ __forceinline__ bool all_valid() const {
+        bool ok = true;
+#pragma unroll
+        for (int i = 0; i < (PLAN == PLAN_STRIDED ? 1 : LOADS); ++i) ok = ok && valid[i];
+        return ok;
     }
 };
 
@@ -273,15 +294,16 @@ struct Ring64x5 {
     template <int P> struct At {
         static constexpr int A_SLAB = (2 * P) % 5, A_OFF = 0, B_SLAB = (2 * P + 1) % 5, B_OFF = 0;
     };
+    static constexpr int LOOKAHEAD = 2;  // a step at stage s issues loads of stages up to s + LOOKAHEAD
     template <typename K> __device__ static __forceinline__ void prologue(K& k) {
-        k.template issue_a<0, 0, L>(0); k.template issue_b<0, 0, L>(0);
-        k.template issue_a<1, 0, L>(1); k.template issue_b<1, 0, H>(1);
+        k.template issue_a<0, 0, L, true>(0); k.template issue_b<0, 0, L, true>(0);
+        k.template issue_a<1, 0, L, true>(1); k.template issue_b<1, 0, H, true>(1);
     }
-    template <int P, int PH, typename K> __device__ static __forceinline__ void issue_phase(K& k, int64_t s) {
-        if constexpr (PH == 0) k.template issue_b<(P + 1) % CYCLE, H, L>(s + 1);
-        else if constexpr (PH == 1) k.template issue_a<(P + 2) % CYCLE, 0, H>(s + 2);
-        else if constexpr (PH == 2) k.template issue_a<(P + 2) % CYCLE, H, L>(s + 2);
-        else k.template issue_b<(P + 2) % CYCLE, 0, H>(s + 2);
+    template <int P, int PH, bool MASKED, typename K> __device__ static __forceinline__ void issue_phase(K& k, int64_t s) {
+        if constexpr (PH == 0) k.template issue_b<(P + 1) % CYCLE, H, L, MASKED>(s + 1);
+        else if constexpr (PH == 1) k.template issue_a<(P + 2) % CYCLE, 0, H, MASKED>(s + 2);
+        else if constexpr (PH == 2) k.template issue_a<(P + 2) % CYCLE, H, L, MASKED>(s + 2);
+        else k.template issue_b<(P + 2) % CYCLE, 0, H, MASKED>(s + 2);
     }
 };
 
@@ -301,11 +323,11 @@ struct Kernel {
     int active_m;            // 32-row blocks of this wave's 128 tile rows that hold existing rows (wave-uniform)
     u32x4_t fa[2][MI], fb[2][NI];  // fragments: the block being multiplied and the one being read
 
-    template <int P, int I0, int I1> __device__ __forceinline__ void issue_a(int64_t stage) {
-        la.template issue<I0, I1>(slab<Pipe::template At<P>::A_SLAB>(), Pipe::template At<P>::A_OFF, stage, red_len);
+    template <int P, int I0, int I1, bool MASKED> __device__ __forceinline__ void issue_a(int64_t stage) {
+        la.template issue<I0, I1, MASKED>(slab<Pipe::template At<P>::A_SLAB>(), Pipe::template At<P>::A_OFF, stage, red_len);
     }
-    template <int P, int I0, int I1> __device__ __forceinline__ void issue_b(int64_t stage) {
-        lb.template issue<I0, I1>(slab<Pipe::template At<P>::B_SLAB>(), Pipe::template At<P>::B_OFF, stage, red_len);
+    template <int P, int I0, int I1, bool MASKED> __device__ __forceinline__ void issue_b(int64_t stage) {
+        lb.template issue<I0, I1, MASKED>(slab<Pipe::template At<P>::B_SLAB>(), Pipe::template At<P>::B_OFF, stage, red_len);
     }
 
     // Byte offsets of this lane's fragments inside an operand tile.  Only the part that is not a
@@ -386,23 +408,23 @@ struct Kernel {
     // branch-free: stages past the end of the reduction fetch the zero page, which keeps the count of loads
     // in flight the same at every step and lets the compiler see that the loop needs no other wait on
     // vector memory.
-    template <int P, int PH, bool FULL>
+    template <int P, int PH, bool FULL, bool MASKED>
     __device__ __forceinline__ void phases_before_barrier(int64_t s, f32x16_t (&acc)[MI][NI]) {
         if constexpr (PH + 1 < Pipe::KK) {
-            Pipe::template issue_phase<P, PH>(*this, s);
+            Pipe::template issue_phase<P, PH, MASKED>(*this, s);
             read_fragments<P, FULL>(PH + 1, fa[(PH + 1) & 1], fb[(PH + 1) & 1]);
             multiply<FULL>(fa[PH & 1], fb[PH & 1], acc);
             if constexpr (FULL) interleave_phase();
-            phases_before_barrier<P, PH + 1, FULL>(s, acc);
+            phases_before_barrier<P, PH + 1, FULL, MASKED>(s, acc);
         }
     }
-    template <int P, bool FULL>
+    template <int P, bool FULL, bool MASKED>
     __device__ __forceinline__ void step(int64_t s, f32x16_t (&acc)[MI][NI]) {
         constexpr int KK = Pipe::KK;
-        phases_before_barrier<P, 0, FULL>(s, acc);
+        phases_before_barrier<P, 0, FULL, MASKED>(s, acc);
         wait_vmcnt_and_lds<Pipe::WAIT>();
         block_barrier();
-        Pipe::template issue_phase<P, KK - 1>(*this, s);
+        Pipe::template issue_phase<P, KK - 1, MASKED>(*this, s);
         read_fragments<(P + 1) % Pipe::CYCLE, FULL>(0, fa[KK & 1], fb[KK & 1]);
         multiply<FULL>(fa[(KK - 1) & 1], fb[(KK - 1) & 1], acc);
         if constexpr (FULL) interleave_phase();
@@ -412,24 +434,28 @@ struct Kernel {
     __device__ __forceinline__ void steps_from(int64_t s, int64_t count, f32x16_t (&acc)[MI][NI]) {
         if constexpr (P < Pipe::CYCLE) {
             if (P < count) {
-                step<P, FULL>(s + P, acc);
+                step<P, FULL, true>(s + P, acc);
                 steps_from<P + 1, FULL>(s, count, acc);
             }
         }
     }
-    template <int P, bool FULL>
+    template <int P, bool FULL, bool MASKED>
     __device__ __forceinline__ void full_cycle(int64_t s, f32x16_t (&acc)[MI][NI]) {
         if constexpr (P < Pipe::CYCLE) {
-            step<P, FULL>(s + P, acc);
-            full_cycle<P + 1, FULL>(s, acc);
+            step<P, FULL, MASKED>(s + P, acc);
+            full_cycle<P + 1, FULL, MASKED>(s, acc);
         }
     }
 
+    // `plain_steps`: the first that many steps only issue loads of stages that lie wholly inside the reduction, in a
+    // tile without missing rows or columns; they take the unmasked form of the loads.
     template <bool FULL>
-    __device__ __forceinline__ void run_stages(int64_t num_stages, f32x16_t (&acc)[MI][NI]) {
+    __device__ __forceinline__ void run_stages(int64_t num_stages, int64_t plain_steps, f32x16_t (&acc)[MI][NI]) {
         read_fragments<0, FULL>(0, fa[0], fb[0]);
         int64_t s = 0;
-        for (; s + Pipe::CYCLE <= num_stages; s += Pipe::CYCLE) full_cycle<0, FULL>(s, acc);
+        if constexpr (FULL)
+            for (; s + Pipe::CYCLE <= plain_steps; s += Pipe::CYCLE) full_cycle<0, FULL, false>(s, acc);
+        for (; s + Pipe::CYCLE <= num_stages; s += Pipe::CYCLE) full_cycle<0, FULL, true>(s, acc);
         steps_from<0, FULL>(s, num_stages - s, acc);  // fewer than CYCLE steps remain
     }
 
@@ -437,23 +463,19 @@ struct Kernel {
         const int64_t num_stages = (red_len + BK - 1) / BK;
         if (num_stages > 0) {
             Pipe::prologue(*this);
-            // Weight-gradient kind: materialise the zeroed accumulators in their registers here, while the first
-            // loads are on their way.  Measured effect on the register allocation of this instantiation: no
-            // accumulator is parked in scratch memory around the last, partial trip round the ring any more
-            // (the row-grouped kinds do not park any, and get worse with the same pin).
-            if constexpr (KIND == XMA_GEMM_MT) {
-#pragma unroll
-                for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) asm volatile("" : "+a"(acc[mi][ni]));
-            }
             wait_vmcnt<Pipe::PROLOGUE_WAIT>();
             block_barrier();
             // The two loops issue the same loads and meet at the same barriers, so waves of one work-group may
             // take different ones.  The row-grouped kinds take the second for the tail tile of an expert's rows:
             // its cost then follows the rows that exist (plus the full weight panel it still has to stream).
-            if (KIND == XMA_GEMM_MT || active_m == MI) run_stages<true>(num_stages, acc);
-            else run_stages<false>(num_stages, acc);
+            if (KIND == XMA_GEMM_MT || active_m == MI) {
+                // wave-uniform: validity is a property of rows and columns of the tile, combined over the lanes
+                const bool whole = __builtin_amdgcn_readfirstlane(__all((int)(la.all_valid() && lb.all_valid()))) != 0;
+                const int64_t plain = whole ? red_len / BK - Pipe::LOOKAHEAD : 0;
+                run_stages<true>(num_stages, plain, acc);
+            } else {
+                run_stages<false>(num_stages, 0, acc);
+            }
             wait_vmcnt<0>();  // the trailing zero-page loads
         }
         block_barrier();  // every wave is done reading the slabs; no load is in flight any more
