@@ -75,6 +75,52 @@ __device__ __forceinline__ void transpose_block<4>(const uint4 (&in)[4], uint4 (
 __device__ __forceinline__ uint4 load16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ __forceinline__ uint4 zero16() { return make_uint4(0u, 0u, 0u, 0u); }
 
+// Element-wise forms of a 16-byte access for operands whose sizes are not multiples of the vector width or whose
+// rows are not 16-byte aligned (the reference's kernels mask such tails,
+// xma/layers/moe/triton_implementation/scatter_kernel.py:39-45,91-95): the first `count` elements are moved one by
+// one, the rest of the vector reads as zero / is not written.
+template <typename T>
+__device__ __forceinline__ uint4 load_elems(const T* p, int count) {
+    constexpr int PV = 16 / (int)sizeof(T);
+    union {
+        uint4 v;
+        T e[PV];
+    } u;
+    u.v = zero16();
+#pragma unroll
+    for (int q = 0; q < PV; ++q)
+        if (q < count) u.e[q] = p[q];
+    return u.v;
+}
+template <typename T>
+__device__ __forceinline__ void store_elems(T* p, const uint4& v, int count) {
+    constexpr int PV = 16 / (int)sizeof(T);
+    union {
+        uint4 v;
+        T e[PV];
+    } u;
+    u.v = v;
+#pragma unroll
+    for (int q = 0; q < PV; ++q)
+        if (q < count) p[q] = u.e[q];
+}
+// number of the PV elements starting at index `first` that lie below `limit`
+__device__ __forceinline__ int elems_below(int64_t first, int64_t limit, int pv) {
+    const int64_t left = limit - first;
+    return left <= 0 ? 0 : left >= pv ? pv : (int)left;
+}
+// RAGGED: element-wise, `count` valid elements; otherwise one vector access (count is 0 or PV)
+template <bool RAGGED, typename T>
+__device__ __forceinline__ uint4 load_vec(const T* p, int count) {
+    if constexpr (RAGGED) return load_elems(p, count);
+    else return count > 0 ? load16(p) : zero16();
+}
+template <bool RAGGED, typename T>
+__device__ __forceinline__ void store_vec(T* p, const uint4& v, int count) {
+    if constexpr (RAGGED) store_elems(p, v, count);
+    else if (count > 0) *reinterpret_cast<uint4*>(p) = v;
+}
+
 // ---- tile loaders -----------------------------------------------------------------------------
 // DirectLoader: the operand's reduction index is contiguous in HBM.  NT threads starting at
 // thread T0 copy R rows x 8 chunks per stage; each thread keeps its chunk column and walks rows.
@@ -101,13 +147,13 @@ struct DirectLoader {
         }
     }
     // k0: first reduction index of the stage, klen: total reduction length
-    template <int NV>
+    template <bool RAGGED, int NV>
     __device__ __forceinline__ void load(uint4 (&v)[NV], int64_t k0, int64_t klen) const {
         static_assert(NV >= ITEMS, "staging registers");
         if (!active) return;
-        const bool k_ok = k0 + chunk * PV < klen;
+        const int count = elems_below(k0 + chunk * PV, klen, PV);
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) v[i] = (row_ptr[i] && k_ok) ? load16(row_ptr[i] + k0) : zero16();
+        for (int i = 0; i < ITEMS; ++i) v[i] = row_ptr[i] ? load_vec<RAGGED>(row_ptr[i] + k0, count) : zero16();
     }
     template <int NV>
     __device__ __forceinline__ void store(const uint4 (&v)[NV], char* lds) const {
@@ -137,16 +183,17 @@ struct TransLoader {
         tcol = lt % TCOLS;
         tk = lt / TCOLS;
     }
-    // ptr_fn(r) returns the HBM address of reduction row (tk*PV + r) of this stage at this thread's
-    // PV tile rows, or nullptr when that row / those tile rows are out of range
-    template <int NV, typename PtrFn>
+    // ptr_fn(r, col, count) returns the HBM address of reduction row (tk*PV + r) of this stage at this thread's
+    // PV tile rows and sets `count` to how many of them exist, or returns nullptr when that row is out of range
+    template <bool RAGGED, int NV, typename PtrFn>
     __device__ __forceinline__ void load(uint4 (&v)[NV], PtrFn ptr_fn) const {
         static_assert(NV >= PV, "staging registers");
         if (!active) return;
 #pragma unroll
         for (int r = 0; r < PV; ++r) {
-            const T* p = ptr_fn(tk * PV + r, tcol * PV);
-            v[r] = p ? load16(p) : zero16();
+            int count = 0;
+            const T* p = ptr_fn(tk * PV + r, tcol * PV, count);
+            v[r] = p ? load_vec<RAGGED>(p, count) : zero16();
         }
     }
     template <int NV>
@@ -161,7 +208,9 @@ struct TransLoader {
     }
 };
 
-template <typename T, int KIND, int EPI>
+// RAGGED: column counts and reduction lengths may be any number and rows may start at any element: every access to
+// HBM is element-wise with per-element bounds (slow, for the shapes the vector forms cannot take).
+template <typename T, int KIND, int EPI, bool RAGGED>
 __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const GemmParams P) {
     using Cfg = TileCfg<T>;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, THREADS = Cfg::THREADS;
@@ -274,27 +323,30 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
 
     auto load_stage = [&](int64_t k0) {
         if constexpr (!A_TRANS) {
-            a_direct.load(st_a, k0, red_len);
+            a_direct.template load<RAGGED>(st_a, k0, red_len);
         } else {
-            a_trans.load(st_a, [&](int r, int col) -> const T* {
+            a_trans.template load<RAGGED>(st_a, [&](int r, int col, int& count) -> const T* {
                 const int64_t p = m_begin + k0 + r;
                 const int64_t i = tile_i0 + col;
-                return (p < m_end && i < P.n) ? A + p * P.lda + i : nullptr;
+                count = elems_below(i, P.n, PV);
+                return (p < m_end && count > 0) ? A + p * P.lda + i : nullptr;
             });
         }
         if constexpr (!B_TRANS) {
-            b_direct.load(st_b, k0, red_len);
+            b_direct.template load<RAGGED>(st_b, k0, red_len);
         } else if constexpr (KIND == XMA_GEMM_NN) {
-            b_trans.load(st_b, [&](int r, int col) -> const T* {
+            b_trans.template load<RAGGED>(st_b, [&](int r, int col, int& count) -> const T* {
                 const int64_t kk = k0 + r;
                 const int64_t n = n0 + col;
-                return (kk < P.k && n < P.n) ? Wexp + kk * P.ldb + n : nullptr;
+                count = elems_below(n, P.n, PV);
+                return (kk < P.k && count > 0) ? Wexp + kk * P.ldb + n : nullptr;
             });
         } else {
-            b_trans.load(st_b, [&](int r, int col) -> const T* {
+            b_trans.template load<RAGGED>(st_b, [&](int r, int col, int& count) -> const T* {
                 const int64_t p = m_begin + k0 + r;
                 const int64_t j = n0 + col;
-                if (p >= m_end || j >= P.k) return nullptr;
+                count = elems_below(j, P.k, PV);
+                if (p >= m_end || count == 0) return nullptr;
                 const int64_t src = P.in_index ? source_row(P, p) : p;
                 return B + src * P.ldb + j;
             });
@@ -394,8 +446,10 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
                         }
                         if (exists) {
                             const T* b = reinterpret_cast<const T*>(P.bias) + (int64_t)expert * P.ld_bias + n;
+                            const int64_t limit = EPI == EPI_PAIRED ? (col >= BN_OUT ? P.n : P.n / 2) : P.n;
 #pragma unroll
-                            for (int q = 0; q < 4; ++q) f[q] += Elem<T>::load(b + q);
+                            for (int q = 0; q < 4; ++q)
+                                if (!RAGGED || n + q < limit) f[q] += Elem<T>::load(b + q);
                         }
                     }
                 }
@@ -418,37 +472,39 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
         const char* src = lds + r * C_ROW_BYTES;
         if constexpr (KIND == XMA_GEMM_MT) {
             const int64_t i = tile_i0 + r, j = n0 + cc * PV;
-            if (i < P.n && j < P.k)
-                *reinterpret_cast<uint4*>(C + (int64_t)expert * P.c_expert_stride + i * P.ldc + j) =
-                    *reinterpret_cast<const uint4*>(src + cc * 16);
+            if (i < P.n)
+                store_vec<RAGGED>(C + (int64_t)expert * P.c_expert_stride + i * P.ldc + j,
+                                  *reinterpret_cast<const uint4*>(src + cc * 16), elems_below(j, P.k, PV));
         } else {
             const int64_t p = m_begin + r;
             if (p >= m_end) break;
             const int64_t orow = P.out_index ? load_index(P.out_index, P.idx_is_i64, p) : p;
             if constexpr (EPI == EPI_PLAIN) {
                 const int64_t n = n0 + cc * PV;
-                if (n < P.n) {
+                const int count = elems_below(n, P.n, PV);
+                if (count > 0) {
                     const uint4 v = *reinterpret_cast<const uint4*>(src + cc * 16);
                     if (KIND == XMA_GEMM_TN && P.act == ACT_GELU_TANH) {
-                        if (P.aux) *reinterpret_cast<uint4*>(reinterpret_cast<T*>(P.aux) + p * P.ld_aux + n) = v;
+                        if (P.aux) store_vec<RAGGED>(reinterpret_cast<T*>(P.aux) + p * P.ld_aux + n, v, count);
                         float h[PV], o[PV];
                         Elem<T>::unpack(v, h);
 #pragma unroll
                         for (int q = 0; q < PV; ++q) o[q] = gelu_tanh_forward<false>(h[q]);
-                        *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = Elem<T>::pack(o);
+                        store_vec<RAGGED>(C + orow * P.ldc + n, Elem<T>::pack(o), count);
                     } else {
-                        *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = v;
+                        store_vec<RAGGED>(C + orow * P.ldc + n, v, count);
                     }
                 }
             } else if constexpr (EPI == EPI_PAIRED) {
                 constexpr int HALF_CHUNKS = C_CHUNKS / 2;
                 const int64_t half = P.n / 2;
                 const int64_t j = n0 + (cc % HALF_CHUNKS) * PV;
-                if (j < half) {
+                const int count = elems_below(j, half, PV);
+                if (count > 0) {
                     if (P.aux) {
                         T* h = reinterpret_cast<T*>(P.aux) + p * P.ld_aux;
-                        *reinterpret_cast<uint4*>(h + (cc < HALF_CHUNKS ? j : half + j)) =
-                            *reinterpret_cast<const uint4*>(src + cc * 16);
+                        store_vec<RAGGED>(h + (cc < HALF_CHUNKS ? j : half + j),
+                                          *reinterpret_cast<const uint4*>(src + cc * 16), count);
                     }
                     if (cc < HALF_CHUNKS) {
                         float u[PV], g[PV], o[PV];
@@ -456,26 +512,27 @@ __global__ __launch_bounds__(TileCfg<T>::THREADS) void grouped_gemm_kernel(const
                         Elem<T>::unpack(*reinterpret_cast<const uint4*>(src + (cc + HALF_CHUNKS) * 16), g);
 #pragma unroll
                         for (int q = 0; q < PV; ++q) o[q] = gated_forward<false>(P.act, u[q], g[q]);
-                        *reinterpret_cast<uint4*>(C + orow * P.ldc + j) = Elem<T>::pack(o);
+                        store_vec<RAGGED>(C + orow * P.ldc + j, Elem<T>::pack(o), count);
                     }
                 }
             } else {  // EPI_BACKWARD: the product is the activation's upstream gradient
                 const int64_t n = n0 + cc * PV;
-                if (n < P.n) {
+                const int count = elems_below(n, P.n, PV);
+                if (count > 0) {
                     const T* h = reinterpret_cast<const T*>(P.aux) + p * P.ld_aux;
                     float u[PV], g[PV], d[PV], du[PV], dg[PV];
-                    Elem<T>::unpack(load16(h + n), u);
+                    Elem<T>::unpack(load_vec<RAGGED>(h + n, count), u);
                     Elem<T>::unpack(*reinterpret_cast<const uint4*>(src + cc * 16), d);
                     if (P.act == ACT_GELU_TANH) {
 #pragma unroll
                         for (int q = 0; q < PV; ++q) du[q] = gelu_tanh_backward<false>(u[q], d[q]);
-                        *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = Elem<T>::pack(du);
+                        store_vec<RAGGED>(C + orow * P.ldc + n, Elem<T>::pack(du), count);
                     } else {
-                        Elem<T>::unpack(load16(h + P.n + n), g);
+                        Elem<T>::unpack(load_vec<RAGGED>(h + P.n + n, count), g);
 #pragma unroll
                         for (int q = 0; q < PV; ++q) gated_backward<false>(P.act, u[q], g[q], d[q], du[q], dg[q]);
-                        *reinterpret_cast<uint4*>(C + orow * P.ldc + n) = Elem<T>::pack(du);
-                        *reinterpret_cast<uint4*>(C + orow * P.ldc + P.n + n) = Elem<T>::pack(dg);
+                        store_vec<RAGGED>(C + orow * P.ldc + n, Elem<T>::pack(du), count);
+                        store_vec<RAGGED>(C + orow * P.ldc + P.n + n, Elem<T>::pack(dg), count);
                     }
                 }
             }
@@ -491,7 +548,7 @@ constexpr int lds_bytes() {
     return stages > ctile ? stages : ctile;
 }
 
-template <typename T, int KIND, int EPI>
+template <typename T, int KIND, int EPI, bool RAGGED>
 static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
     using Cfg = TileCfg<T>;
     constexpr int PV = Elem<T>::kPerVec;
@@ -519,7 +576,7 @@ static int launch(const xma_grouped_gemm_args& a, hipStream_t stream) {
     }
     XMA_REQUIRE(grid < ((int64_t)1 << 31), "xma_grouped_gemm: %lld tiles exceed the grid limit", (long long)grid);
     (void)PV;
-    auto kernel = grouped_gemm_kernel<T, KIND, EPI>;
+    auto kernel = grouped_gemm_kernel<T, KIND, EPI, RAGGED>;
     // set on every launch: the attribute belongs to the (function, device) pair, and the call is a cheap host-side
     // update that needs no shared flag between threads
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -563,20 +620,24 @@ void fill_params(const xma_grouped_gemm_args& a, GemmParams& P) {
     P.col_tiles = 0;
 }
 
-template <typename T>
+template <typename T, bool RAGGED>
 static int dispatch_kind(const xma_grouped_gemm_args& a, hipStream_t stream) {
     int shape = EPI_PLAIN, act = ACT_NONE;
     split_epilogue(a.epilogue, shape, act);
     switch (a.kind) {
         case XMA_GEMM_TN:
-            if (shape == EPI_PAIRED) return launch<T, XMA_GEMM_TN, EPI_PAIRED>(a, stream);
-            return launch<T, XMA_GEMM_TN, EPI_PLAIN>(a, stream);
+            if (shape == EPI_PAIRED) return launch<T, XMA_GEMM_TN, EPI_PAIRED, RAGGED>(a, stream);
+            return launch<T, XMA_GEMM_TN, EPI_PLAIN, RAGGED>(a, stream);
         case XMA_GEMM_NN:
-            if (shape == EPI_BACKWARD) return launch<T, XMA_GEMM_NN, EPI_BACKWARD>(a, stream);
-            return launch<T, XMA_GEMM_NN, EPI_PLAIN>(a, stream);
+            if (shape == EPI_BACKWARD) return launch<T, XMA_GEMM_NN, EPI_BACKWARD, RAGGED>(a, stream);
+            return launch<T, XMA_GEMM_NN, EPI_PLAIN, RAGGED>(a, stream);
         default:
-            return launch<T, XMA_GEMM_MT, EPI_PLAIN>(a, stream);
+            return launch<T, XMA_GEMM_MT, EPI_PLAIN, RAGGED>(a, stream);
     }
+}
+template <typename T>
+static int dispatch_kind(const xma_grouped_gemm_args& a, bool ragged, hipStream_t stream) {
+    return ragged ? dispatch_kind<T, true>(a, stream) : dispatch_kind<T, false>(a, stream);
 }
 
 static int largest_bm() { return TileCfg<bf16_t>::BM > TileCfg<float>::BM ? TileCfg<bf16_t>::BM : TileCfg<float>::BM; }
@@ -615,14 +676,18 @@ int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
                 a.num_experts);
     XMA_REQUIRE(a.rows >= 0 && a.rows < ((int64_t)1 << 31) && a.n >= 0 && a.k >= 0, "xma_grouped_gemm: bad sizes");
     XMA_REQUIRE(a.expert_offsets != nullptr, "xma_grouped_gemm: expert_offsets is null");
+    // Sizes that are multiples of the vector width (8 elements of a 16-bit type, 4 of fp32) and 16-byte aligned rows
+    // take the vector kernels.  Anything else takes the element-wise form of the register-staged kernel: correct for
+    // every size and alignment, at a fraction of the speed.
     const int pv = a.dtype == XMA_F32 ? 4 : 8;
-    XMA_REQUIRE(a.n % pv == 0 && a.k % pv == 0, "xma_grouped_gemm: n=%lld and k=%lld must be multiples of %d",
-                (long long)a.n, (long long)a.k, pv);
-    XMA_REQUIRE(a.lda % pv == 0 && a.ldb % pv == 0 && a.ldc % pv == 0 && a.b_expert_stride % pv == 0 &&
-                    a.c_expert_stride % pv == 0 && a.ld_aux % pv == 0,
-                "xma_grouped_gemm: strides must keep rows 16-byte aligned");
-    XMA_REQUIRE(aligned16(a.a) && aligned16(a.b) && aligned16(a.c) && aligned16(a.aux),
-                "xma_grouped_gemm: operands must be 16-byte aligned");
+    const int64_t elem = a.dtype == XMA_F32 ? 4 : 2;
+    auto elem_aligned = [&](const void* p) { return (reinterpret_cast<uintptr_t>(p) % elem) == 0; };
+    XMA_REQUIRE(elem_aligned(a.a) && elem_aligned(a.b) && elem_aligned(a.c) && elem_aligned(a.aux) && elem_aligned(a.bias),
+                "xma_grouped_gemm: operands must be aligned to their element size");
+    const bool ragged = a.n % pv != 0 || a.k % pv != 0 || a.lda % pv != 0 || a.ldb % pv != 0 || a.ldc % pv != 0 ||
+                        a.b_expert_stride % pv != 0 || a.c_expert_stride % pv != 0 || a.ld_aux % pv != 0 ||
+                        (a.bias != nullptr && a.ld_bias % pv != 0) || !aligned16(a.a) || !aligned16(a.b) ||
+                        !aligned16(a.c) || !aligned16(a.aux) || !aligned16(a.bias);
     const bool mt = a.kind == XMA_GEMM_MT;
     if (mt) {
         XMA_REQUIRE(a.epilogue == XMA_EPI_NONE && a.bias == nullptr, "xma_grouped_gemm: MT takes no epilogue and no bias");
@@ -644,7 +709,7 @@ int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
         XMA_REQUIRE(a.lda >= a.k, "xma_grouped_gemm: lda too small");
         XMA_REQUIRE(a.ldb >= (a.kind == XMA_GEMM_TN ? a.k : a.n), "xma_grouped_gemm: ldb too small");
         if (shape == EPI_PAIRED) {
-            XMA_REQUIRE(a.n % (2 * pv) == 0, "xma_grouped_gemm: gated epilogue needs n %% %d == 0", 2 * pv);
+            XMA_REQUIRE(a.n % 2 == 0, "xma_grouped_gemm: gated epilogue needs an even n");
             XMA_REQUIRE(a.ldc >= a.n / 2, "xma_grouped_gemm: ldc too small");
             XMA_REQUIRE(a.aux == nullptr || a.ld_aux >= a.n, "xma_grouped_gemm: ld_aux too small");
         } else if (shape == EPI_BACKWARD) {
@@ -658,8 +723,8 @@ int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
             XMA_REQUIRE(act == ACT_NONE || a.out_index == nullptr || a.aux == nullptr,
                         "xma_grouped_gemm: the pre-activation is kept for grouped outputs only");
         }
-        XMA_REQUIRE(a.bias == nullptr || (a.kind == XMA_GEMM_TN && a.ld_bias >= a.n && a.ld_bias % pv == 0 && aligned16(a.bias)),
-                    "xma_grouped_gemm: bias needs a forward (TN) kind, ld_bias >= n and 16-byte aligned rows");
+        XMA_REQUIRE(a.bias == nullptr || (a.kind == XMA_GEMM_TN && a.ld_bias >= a.n),
+                    "xma_grouped_gemm: bias needs a forward (TN) kind and ld_bias >= n");
         if (a.rows == 0 || a.n == 0) return 0;
         XMA_REQUIRE(a.workspace != nullptr &&
                         a.workspace_bytes >= xma_grouped_gemm_workspace_bytes(a.num_experts, a.rows),
@@ -668,14 +733,17 @@ int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
     }
     XMA_REQUIRE(a.a && a.b && a.c, "xma_grouped_gemm: null operand");
     hipStream_t stream = (hipStream_t)stream_;
-    if (dma_gemm_supports(a)) return launch_dma_gemm(a, stream);
+    // a gated tile of the vector kernels pairs whole 16-byte chunks of the two halves
+    const bool paired_tail = (a.epilogue == XMA_EPI_SWIGLU || a.epilogue == XMA_EPI_GLU) && a.n % (2 * pv) != 0;
+    const bool elementwise = ragged || paired_tail;
+    if (!elementwise && dma_gemm_supports(a)) return launch_dma_gemm(a, stream);
     switch (a.dtype) {
         case XMA_F32:
-            return dispatch_kind<float>(a, stream);
+            return dispatch_kind<float>(a, elementwise, stream);
         case XMA_F16:
-            return dispatch_kind<f16_t>(a, stream);
+            return dispatch_kind<f16_t>(a, elementwise, stream);
         default:
-            return dispatch_kind<bf16_t>(a, stream);
+            return dispatch_kind<bf16_t>(a, elementwise, stream);
     }
 }
 

@@ -34,6 +34,8 @@ CASES = [
     (1000, 576, 264, 32, 4, (2, 31)),  # K tail (264 = 4*64 + 8), N not a tile multiple
     (2048, 1024, 512, 8, 2, (0,)),
     (513, 200, 104, 5, 3, (4,)),
+    (300, 100, 52, 4, 2, ()),  # neither H nor I a multiple of the vector width: the element-wise kernel
+    (129, 66, 35, 3, 2, (1,)),  # odd I: rows of the activation start at odd elements
 ]
 
 
@@ -249,12 +251,15 @@ def test_argument_validation():
     off = torch.tensor([0, 8, 8], device=dev, dtype=torch.int32)
     out = torch.empty(8, 32, device=dev, dtype=torch.bfloat16)
     ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, out, 1, False, True, off)  # sanity: valid call
-    with pytest.raises(RuntimeError, match="multiples"):
-        bad_w = torch.randn(2, 12, 64, device=dev, dtype=torch.bfloat16)
-        ops.scatter2scatter(x, bad_w.permute(0, 2, 1), se, idx, out[:, :12], 1, False, True, off)
-    with pytest.raises(RuntimeError, match="aligned"):
-        shifted = torch.randn(8 * 64 + 8, device=dev, dtype=torch.bfloat16)[1 : 1 + 8 * 64].view(8, 64)
-        ops.scatter2scatter(shifted, w.permute(0, 2, 1), se, idx, out, 1, False, True, off)
+    # column counts that are not multiples of the vector width and rows that are not 16-byte aligned are served by
+    # the element-wise kernel (the reference masks such tails, scatter_kernel.py:39-45)
+    bad_w = torch.randn(2, 12, 64, device=dev, dtype=torch.bfloat16)
+    narrow = torch.full((8, 12), float("nan"), device=dev, dtype=torch.bfloat16)
+    ops.scatter2scatter(x, bad_w.permute(0, 2, 1), se, idx, narrow, 1, False, True, off)
+    assert_close(narrow, x.float() @ bad_w[0].float().T, TOL[torch.bfloat16], "12 output columns")
+    shifted = torch.randn(8 * 64 + 8, device=dev, dtype=torch.bfloat16)[1 : 1 + 8 * 64].view(8, 64)
+    ops.scatter2scatter(shifted, w.permute(0, 2, 1), se, idx, out, 1, False, True, off)
+    assert_close(out, shifted.float() @ w[0].float().T, TOL[torch.bfloat16], "rows that start at an odd element")
     with pytest.raises(AssertionError):
         ops.scatter2scatter(x, w.permute(0, 2, 1), se, idx, out, 1, False, True, off[:1])  # neither E nor E + 1 long
     with pytest.raises(ValueError):

@@ -136,6 +136,17 @@ def test_fine_grained_reduced():
     _run_case(2048, 512, 256, 64, 6, torch.bfloat16)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("activation", ["swiglu", "gelu"])
+def test_sizes_that_are_not_multiples_of_the_vector_width(activation, dtype):
+    """hidden 100, intermediate 52 (and an odd pair, 66 / 35): no dimension is a multiple of 8, rows of every
+    intermediate start at unaligned addresses.  The reference's kernels mask such tails
+    (scatter_kernel.py:39-45,91-95,134; group_backward_kernel.py:62-66,77-91,99)."""
+
+    _run_case(333, 100, 52, 6, 2, dtype, activation=activation, seed=5)
+    _run_case(77, 66, 35, 4, 3, dtype, activation=activation, seed=6, few_rows=True)
+
+
 def test_skewed_routing_reduced():
     """Zipf(1.2) bias over the expert index: overloaded, ragged and empty groups."""
 

@@ -72,10 +72,10 @@ def test_identification_and_error_channel():
     assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "struct_size" in _native.last_error()
     args.struct_size = ctypes.sizeof(args)
     assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "num_experts" in _native.last_error()
-    args.num_experts, args.n, args.k = 4, 12, 64  # n not a multiple of 8
+    args.num_experts, args.n, args.k, args.lda = 4, 12, 64, 32  # row stride of A shorter than the reduction
     off = (ctypes.c_int32 * 5)()
     args.expert_offsets = ctypes.cast(off, ctypes.c_void_p)
-    assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "multiples" in _native.last_error()
+    assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "lda too small" in _native.last_error()
     assert lib.xma_grouped_gemm(None, None) != 0
     assert lib.xma_route_workspace_bytes(1 << 20, 256) == (1 << 20) // 1024 * 256 * 4
     assert lib.xma_grouped_gemm_workspace_bytes(8, 16384) >= (4 + 2 * (16384 // 128 + 8)) * 4
