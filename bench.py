@@ -24,6 +24,8 @@ if ROOT not in sys.path:
 
 # MI355X published peaks (dense)
 PEAK_BF16_FLOPS = 2.5e15
+PEAK_FP16_FLOPS = 2.5e15
+PEAK_FP32_MATRIX_FLOPS = 157.3e12
 PEAK_HBM_BYTES = 8.0e12
 
 # HBM-side bytes per launch of the grouped GEMM kernels at this workload are not measured by this script: they come
@@ -37,6 +39,19 @@ TRAFFIC_ROW_TAGS = {
     (1, 2): "xma_grouped_gemm/NN+swiglu_bwd",
     (1, 0): "xma_grouped_gemm/NN",
 }
+
+
+def _profile_blob_id() -> str | None:
+    """git blob id (sha1 of 'blob <size>\\0' + contents) of the profile summary the traffic figure is read from, so
+    that a reader can tell which revision of the file a result line used; None if the file is absent."""
+
+    import hashlib
+
+    try:
+        data = open(os.path.join(ROOT, TRAFFIC_PROFILE), "rb").read()
+    except OSError:
+        return None
+    return hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest()
 
 
 def _profiled_traffic_bytes() -> dict:
@@ -98,6 +113,10 @@ def _parse() -> argparse.Namespace:
     ap.add_argument("--no-aux", action="store_true", help="skip the stand-alone timings of the HBM-bound kernels")
     ap.add_argument("--no-other-configs", action="store_true", help="skip the fine-grained and skewed-routing layers")
     ap.add_argument("--other-steps", type=int, default=10, help="timed passes of each of the other configurations")
+    ap.add_argument("--no-other-dtypes", action="store_true", help="skip the fp16 and fp32 passes of the same layer")
+    ap.add_argument("--no-library-gemm", action="store_true", help="skip the loop of library GEMMs of the same shapes")
+    ap.add_argument("--library-gemm-only", action="store_true",
+                    help="run only the loop of library GEMMs (the command the library's counter profile is taken with)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument(
         "--copy-probe",
@@ -246,6 +265,108 @@ def _other_config(workload: dict, steps: int, warmup: int) -> dict:
     return result
 
 
+def _other_dtype(dtype_name: str, steps: int, warmup: int) -> dict:
+    """The headline layer (same shape, same seed) in another element type: fp16 through the same LDS-DMA kernels as
+    bf16, fp32 through the register-staged kernel with true-fp32 matrix instructions.  Timed like the headline region."""
+
+    import torch
+
+    import flash_model_architectures_amd as xma
+    from flash_model_architectures_amd import _native
+
+    dt, peak = {"fp16": (torch.float16, PEAK_FP16_FLOPS), "fp32": (torch.float32, PEAK_FP32_MATRIX_FLOPS)}[dtype_name]
+    dev = torch.device("cuda:0")
+    T, H, I = WORKLOAD["tokens"], WORKLOAD["hidden"], WORKLOAD["intermediate"]
+    E, k = WORKLOAD["experts"], WORKLOAD["top_k"]
+    torch.manual_seed(0)
+    moe = xma.MoE(E, k, H, I, xma.swiglu_packed, True, False, 0.02).to(dt).to(dev)
+    x = torch.randn(T, H, device=dev).to(dt).requires_grad_()
+    d_y = torch.randn(T, H, device=dev).to(dt)
+
+    def step() -> None:
+        y, _ = moe(x)
+        y.backward(d_y)
+        x.grad = None
+        moe.zero_grad(set_to_none=True)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    timeline = _native.Timeline()
+    _native.set_timeline(timeline)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    _native.set_timeline(None)
+    kernels = _kernel_table(timeline.summary(), steps)
+    for kr in kernels:  # the table's fraction column assumes the bf16 peak
+        if "tflops" in kr:
+            kr["frac_of_matrix_peak"] = round(kr["tflops"] * 1e12 / peak, 4)
+            kr.pop("frac_of_bf16_peak", None)
+    gemm_ms = sum(kr["ms_per_step"] for kr in kernels if kr["kernel"].startswith("xma_grouped_gemm"))
+    flops = 18.0 * T * k * H * I
+    ms_per_step = seconds / steps * 1e3
+    return {
+        "dtype": dtype_name,
+        "matrix_peak_tflops": peak / 1e12,
+        "tokens_per_s": round(T * steps / seconds, 1),
+        "ms_per_step": round(ms_per_step, 3),
+        "steps": steps,
+        "grouped_gemm_ms_per_step": round(gemm_ms, 4),
+        "grouped_gemm_tflops": round(flops / (gemm_ms * 1e-3) / 1e12, 2) if gemm_ms else None,
+        "grouped_gemm_frac_of_matrix_peak": round(flops / (gemm_ms * 1e-3) / peak, 4) if gemm_ms else None,
+        "kernels": [kr for kr in kernels if kr["kernel"].startswith("xma_grouped_gemm")],
+    }
+
+
+def _library_gemms(T: int, H: int, I: int, E: int, k: int, iters: int = 3) -> dict:
+    """The six GEMM groups of a pass as a loop of LIBRARY GEMMs (torch.matmul -> hipBLASLt), one per expert, every
+    expert holding M / E rows, random bf16 operands: no ragged groups, no gather / scatter, no fused activation.  A
+    comparison figure for the grouped kernels, measured on the same device in the same run."""
+
+    import torch
+
+    dev, dt = "cuda", torch.bfloat16
+    rows = T * k // E
+    g = torch.Generator(device=dev).manual_seed(1)
+    mk = lambda *shape: torch.randn(*shape, device=dev, generator=g).to(dt)
+    x, a, dy, dh = mk(rows, H), mk(rows, I), mk(rows, H), mk(rows, 2 * I)
+    w1, w2 = mk(E, 2 * I, H), mk(E, H, I)
+    groups = {
+        "up projection [M/E,H] x [2I,H]^T": (lambda e: torch.matmul(x, w1[e].t()), 2.0 * rows * 2 * I * H),
+        "down projection [M/E,I] x [H,I]^T": (lambda e: torch.matmul(a, w2[e].t()), 2.0 * rows * I * H),
+        "d act [M/E,H] x [H,I]": (lambda e: torch.matmul(dy, w2[e]), 2.0 * rows * I * H),
+        "dX [M/E,2I] x [2I,H]": (lambda e: torch.matmul(dh, w1[e]), 2.0 * rows * 2 * I * H),
+        "dW up [M/E,2I]^T x [M/E,H]": (lambda e: torch.matmul(dh.t(), x), 2.0 * rows * 2 * I * H),
+        "dW down [M/E,H]^T x [M/E,I]": (lambda e: torch.matmul(dy.t(), a), 2.0 * rows * I * H),
+    }
+    out, total_ms, total_flops = [], 0.0, 0.0
+    for name, (fn, flops) in groups.items():
+        for e in range(E):
+            fn(e)
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            for e in range(E):
+                fn(e)
+        end.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(end) / iters
+        total_ms += ms
+        total_flops += flops * E
+        out.append({"gemm": name, "ms_all_experts": round(ms, 4), "tflops": round(flops * E / ms / 1e9, 1),
+                    "frac_of_bf16_peak": round(flops * E / (ms * 1e-3) / PEAK_BF16_FLOPS, 4)})
+    return {
+        "what": f"{E} library GEMMs per group, {rows} rows each, bf16, random operands (torch.matmul)",
+        "ms_per_pass": round(total_ms, 3),
+        "frac_of_bf16_peak": round(total_flops / (total_ms * 1e-3) / PEAK_BF16_FLOPS, 4),
+        "groups": out,
+    }
+
+
 def _aux_hbm_kernels(T: int, H: int, I: int, E: int, k: int) -> list:
     """Stand-alone timings (events on the current stream, outside the timed steps) of the HBM-bound kernels of
     the path at this workload's sizes, plus the histogram / permutation / row moves at fixed large sizes
@@ -324,6 +445,10 @@ def main() -> int:
     E, k = WORKLOAD["experts"], WORKLOAD["top_k"]
     dt = torch.bfloat16
 
+    if args.library_gemm_only:
+        print(json.dumps({"library_gemm": _library_gemms(T, H, I, E, k, iters=max(args.steps, 1))}))
+        return 0
+
     moe = xma.MoE(E, k, H, I, xma.swiglu_packed, True, False, 0.02).to(dt).to(dev)
     x = torch.randn(T, H, device=dev).to(dt).requires_grad_()
     d_y = torch.randn(T, H, device=dev).to(dt)
@@ -372,6 +497,7 @@ def main() -> int:
             "traffic": _profiled_traffic_bytes().get(dominant["kernel"]),
             "traffic_source": TRAFFIC_PROFILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script; "
             "read from that file, not measured in this run)",
+            "traffic_profile_blob": _profile_blob_id(),
             "algorithmic_flops_per_launch": dominant["flops_per_launch"],
         }
     else:
@@ -408,6 +534,10 @@ def main() -> int:
     }
     if not args.no_other_configs:
         result["other_configs"] = [_other_config(w, args.other_steps, 2) for w in OTHER_WORKLOADS]
+    if not args.no_other_dtypes:
+        result["other_dtypes"] = [_other_dtype("fp16", 5, 2), _other_dtype("fp32", 2, 1)]
+    if not args.no_library_gemm:
+        result["library_gemm"] = _library_gemms(T, H, I, E, k)
     if not args.no_aux:
         result["aux_hbm_kernels"] = _aux_hbm_kernels(T, H, I, E, k)
     if not args.no_cpu_baseline:
