@@ -115,6 +115,8 @@ def _parse() -> argparse.Namespace:
     ap.add_argument("--other-steps", type=int, default=10, help="timed passes of each of the other configurations")
     ap.add_argument("--no-other-dtypes", action="store_true", help="skip the fp16 and fp32 passes of the same layer")
     ap.add_argument("--no-library-gemm", action="store_true", help="skip the loop of library GEMMs of the same shapes")
+    ap.add_argument("--only-config", choices=["fine-grained", "skewed"], default=None,
+                    help="run only that one of the other configurations (the command its profile is taken with)")
     ap.add_argument("--library-gemm-only", action="store_true",
                     help="run only the loop of library GEMMs (the command the library's counter profile is taken with)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
@@ -359,11 +361,31 @@ def _library_gemms(T: int, H: int, I: int, E: int, k: int, iters: int = 3) -> di
         total_flops += flops * E
         out.append({"gemm": name, "ms_all_experts": round(ms, 4), "tflops": round(flops * E / ms / 1e9, 1),
                     "frac_of_bf16_peak": round(flops * E / (ms * 1e-3) / PEAK_BF16_FLOPS, 4)})
+    # and ONE dense GEMM per projection over all M routed rows with a single expert's weights: the same FLOPs as the
+    # grouped launch with no group structure at all, i.e. what the library reaches when nothing is ragged
+    xa, aa = mk(T * k, H), mk(T * k, I)
+    dense = []
+    for name, fn, flops in (
+        ("dense [M,H] x [2I,H]^T", lambda: torch.matmul(xa, w1[0].t()), 2.0 * T * k * 2 * I * H),
+        ("dense [M,I] x [H,I]^T", lambda: torch.matmul(aa, w2[0].t()), 2.0 * T * k * I * H),
+    ):
+        fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(end) / iters
+        dense.append({"gemm": name, "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                      "frac_of_bf16_peak": round(flops / (ms * 1e-3) / PEAK_BF16_FLOPS, 4)})
     return {
         "what": f"{E} library GEMMs per group, {rows} rows each, bf16, random operands (torch.matmul)",
         "ms_per_pass": round(total_ms, 3),
         "frac_of_bf16_peak": round(total_flops / (total_ms * 1e-3) / PEAK_BF16_FLOPS, 4),
         "groups": out,
+        "single_dense_gemm_of_the_same_size": dense,
     }
 
 
@@ -445,6 +467,10 @@ def main() -> int:
     E, k = WORKLOAD["experts"], WORKLOAD["top_k"]
     dt = torch.bfloat16
 
+    if args.only_config is not None:
+        workload = OTHER_WORKLOADS[0 if args.only_config == "fine-grained" else 1]
+        print(json.dumps({"other_configs": [_other_config(workload, args.other_steps, 2)]}))
+        return 0
     if args.library_gemm_only:
         print(json.dumps({"library_gemm": _library_gemms(T, H, I, E, k, iters=max(args.steps, 1))}))
         return 0

@@ -607,10 +607,22 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         if (work.parts > 1) {
             // The parts of a tile run on different XCDs, whose L2 caches are not kept coherent with each other.  Fences
             // at device scope would do (each writes back and invalidates the XCD's whole L2, once per wave, under
-            // every other work-group of the XCD: 150-200 k cycles per exchange, measured); instead the partial sums
-            // and the arrival counter are accessed with relaxed device-scope atomics, which go through to memory by
-            // themselves, and what orders them is that every wave's stores have completed before the barrier that
-            // precedes the arrival.
+            // every other work-group of the XCD: 150-200 k cycles per exchange, measured).  Instead the partial sums
+            // and the arrival counter are accessed with relaxed DEVICE-SCOPE ATOMIC stores, loads and one
+            // read-modify-write.  What the exchange relies on, and where each piece comes from:
+            //   (1) a device-scope atomic access is performed at the level of the memory hierarchy that all XCDs
+            //       share, never out of an XCD's private L2: the gfx942/gfx950 memory model of the compiler gives such
+            //       accesses the sc1 bit for exactly that reason (atomicity across the XCDs of one device);
+            //   (2) `s_waitcnt vmcnt(0)` returns when every earlier vector-memory access of the wave, stores
+            //       included, has been acknowledged by the level that performs it;
+            //   (3) the work-group barrier (with its release / acquire fences at work-group scope, which also stop
+            //       the compiler from moving memory accesses across it) orders the four waves: when thread 0 counts
+            //       the arrival, all partial sums of the work-group have been performed;
+            //   (4) the read-modify-write on the counter is performed at the same shared level, so the part that
+            //       reads parts - 1 comes after every other part's sums; its loads, device-scope atomics again, are
+            //       issued after a further work-group barrier and cannot be satisfied from a stale line of its L2.
+            // The compiler cannot reorder any of this: the waits carry memory clobbers, the barriers are fences, and
+            // atomics are never merged, widened or hoisted across them.
             auto part_buffer = [&](int part) {
                 return reinterpret_cast<uint64_t*>(P.split_partials +
                                                    (int64_t)(part * work.split_tiles + work.split_tile) * kSplitTileFloats);
