@@ -9,10 +9,14 @@ namespace xma {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // 16 bytes moved as ONE vector access
 
 constexpr int kNumXcd = 8;     // accelerator complex dies, each with a private L2
-constexpr int kBandTiles = 4;  // row tiles per band of the tile walk
+#ifndef XMA_BAND_TILES
+#define XMA_BAND_TILES 4
+#endif
+constexpr int kBandTiles = XMA_BAND_TILES;  // row tiles per band of the tile walk
 
 // ---- kernel arguments -----------------------------------------------------------------------------
 struct GemmParams {
@@ -266,6 +270,27 @@ struct Mma<bf16_t> {
     __device__ static __forceinline__ void run(const V& x, const V& y, f32x16_t& acc) {
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, x), __builtin_bit_cast(bf16x8_t, y),
                                                       acc, 0, 0, 0);
+    }
+};
+// The 16x16x32 form: acc(16x16) += X(16 x 32) * Y(16 x 32)^T; lane l supplies row l%16 and the 8 reduction
+// elements 8*(l/16)..+7 of both operands; result register r of lane l is D[4*(l/16) + r][l%16] (rows from X).  Half the
+// accumulator traffic per FLOP of the 32x32x16 form: under the device's power cap it sustains a higher clock.  Written
+// as inline assembly with the accumulator tied in place: the compiler's builtin has no tied form for a four-register
+// result and copies accumulators once all 256 are live.
+template <typename T>
+struct Mma16;
+template <>
+struct Mma16<bf16_t> {
+    template <typename V>
+    __device__ static __forceinline__ void run(const V& x, const V& y, f32x4_t& acc) {
+        asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
+    }
+};
+template <>
+struct Mma16<f16_t> {
+    template <typename V>
+    __device__ static __forceinline__ void run(const V& x, const V& y, f32x4_t& acc) {
+        asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
     }
 };
 template <>

@@ -33,7 +33,8 @@ namespace xma {
 namespace dma {
 
 constexpr int BM = 256, BN = 256, THREADS = 256, NUM_WAVES = THREADS / 64;
-constexpr int WAVES_N = 2, WM = 128, WN = 128, MI = WM / 32, NI = WN / 32;
+constexpr int WAVES_N = 2, WM = 128, WN = 128, MI = WM / 16, NI = WN / 16;  // 8 x 8 blocks of 16 x 16 per wave
+constexpr int OUT_SLABS = 4;  // the epilogue stages the tile through LDS 64 rows (one slab) at a time
 constexpr int SLAB_BYTES = 32768;
 static_assert(BM == BN, "both operands use the same tile height");
 
@@ -119,20 +120,20 @@ struct Geometry {
 
     __device__ static __forceinline__ int swizzle(int row) { return BK == 32 ? (row >> 2) & 3 : (row >> 1) & 7; }
 
-    // K-contiguous tile: byte offset of the fragment (row, reduction elements kk*16 + 8*half .. +7)
-    __device__ static __forceinline__ int kcontig_offset(int row, int kk, int half) {
-        return row * ROW_BYTES + (((2 * kk + half) ^ swizzle(row)) << 4);
+    // K-contiguous tile: byte offset of the fragment (row, reduction elements kb*32 + 8*quarter .. +7)
+    __device__ static __forceinline__ int kcontig_offset(int row, int kb, int quarter) {
+        return row * ROW_BYTES + (((4 * kb + quarter) ^ swizzle(row)) << 4);
     }
     // K-strided tile: byte offset of the first of the two transposing reads of the fragment
-    // (tile rows col0..col0+31, reduction elements kk*16 .. +15).  Within each 16-lane group the
+    // (tile rows col0..col0+15, reduction elements kb*32 .. +31).  Within each 16-lane group the
     // instruction hands lane i the i-th 16-bit element of four 16-element rows, where row j is assembled
-    // from the 8-byte pieces addressed by lanes 4j..4j+3.  So lane i addresses (k row i/4, columns
-    // 4*(i%4)..+3) and receives four consecutive k of column i; a second read four k rows further down
-    // completes the eight reduction elements of the MFMA operand.
-    __device__ static __forceinline__ int kstrided_offset(int col0, int kk, int lane) {
+    // from the 8-byte pieces addressed by lanes 4j..4j+3.  So lane i of group g addresses (k row 8g + i/4,
+    // columns 4*(i%4)..+3) and receives four consecutive k of column i; a second read four k rows further
+    // down completes the eight reduction elements 8g .. 8g+7 of the MFMA operand.
+    __device__ static __forceinline__ int kstrided_offset(int col0, int kb, int lane) {
         const int i = lane & 15, group = lane >> 4;
-        const int col = col0 + 16 * (group & 1) + 4 * (i & 3);
-        const int krow0 = kk * 16 + 8 * (group >> 1) + (i >> 2);
+        const int col = col0 + 4 * (i & 3);
+        const int krow0 = kb * 32 + 8 * group + (i >> 2);
         const int chunk = (col >> 3) ^ ((krow0 & 3) << 2);  // (krow0 + 4) & 3 == krow0 & 3
         return krow0 * (BN * 2) + (chunk << 4) + ((col & 4) << 1);
     }
@@ -280,30 +281,30 @@ struct OperandLoads {
 // unit takes about sixteen cycles per DMA instruction and a wave that issues into a full queue stalls,
 // matrix instructions included.
 //
-// Ring64x5: stage j of 64 reduction elements keeps its A tile in slab (2j) % 5 and its B tile in slab
-// (2j + 1) % 5, so every DMA instruction of a K-contiguous operand asks for whole 128-byte lines.  At a
-// step's barrier the next stage has landed and the A tile of the one after is in flight.  The step's own
-// slabs then take the B tile of stage s+2 (half after the barrier, half in the next step's first phase)
-// and the A tile of stage s+3 (second and third phase of the next step).
+// Ring64x5: stage j of 64 reduction elements (two phases of 32) keeps its A tile in slab (2j) % 5 and its B tile
+// in slab (2j + 1) % 5, so every DMA instruction of a K-contiguous operand asks for whole 128-byte lines.  At a
+// step's barrier the next stage has landed and the A tile of the one after is in flight.  The step's own slabs then
+// take the B tile of stage s+2 (during the rest of the step) and the A tile of stage s+3 (during the first phase of
+// the next step): every load is issued between one and a half and two and a half phases before the barrier that
+// needs it.
 struct Ring64x5 {
-    static constexpr int BK = 64, CYCLE = 5, KK = 4;
-    static constexpr int L = Geometry<BK>::LOADS, H = L / 2;
-    static constexpr int PHASE_LOADS = H;
-    static constexpr int WAIT = L;
-    static constexpr int PROLOGUE_WAIT = L + H;
+    static constexpr int BK = 64, CYCLE = 5, KK = 2;
+    static constexpr int L = Geometry<BK>::LOADS;
+    static constexpr int PHASE_LOADS = L;
+    static constexpr int WAIT = L;               // loads that may stay in flight at a step's barrier
+    static constexpr int PROLOGUE_WAIT = 2 * L;  // ... and when the first stage is needed
     template <int P> struct At {
         static constexpr int A_SLAB = (2 * P) % 5, A_OFF = 0, B_SLAB = (2 * P + 1) % 5, B_OFF = 0;
     };
     static constexpr int LOOKAHEAD = 2;  // a step at stage s issues loads of stages up to s + LOOKAHEAD
     template <typename K> __device__ static __forceinline__ void prologue(K& k) {
         k.template issue_a<0, 0, L, true>(0); k.template issue_b<0, 0, L, true>(0);
-        k.template issue_a<1, 0, L, true>(1); k.template issue_b<1, 0, H, true>(1);
+        k.template issue_a<1, 0, L, true>(1); k.template issue_b<1, 0, L, true>(1);
     }
-    template <int P, int PH, bool MASKED, typename K> __device__ static __forceinline__ void issue_phase(K& k, int64_t s) {
-        if constexpr (PH == 0) k.template issue_b<(P + 1) % CYCLE, H, L, MASKED>(s + 1);
-        else if constexpr (PH == 1) k.template issue_a<(P + 2) % CYCLE, 0, H, MASKED>(s + 2);
-        else if constexpr (PH == 2) k.template issue_a<(P + 2) % CYCLE, H, L, MASKED>(s + 2);
-        else k.template issue_b<(P + 2) % CYCLE, 0, H, MASKED>(s + 2);
+    // load number I (0 <= I < PHASE_LOADS) of phase PH of the step at ring position P on stage s
+    template <int P, int PH, int I, bool MASKED, typename K> __device__ static __forceinline__ void issue_one(K& k, int64_t s) {
+        if constexpr (PH == 0) k.template issue_a<(P + 2) % CYCLE, I, I + 1, MASKED>(s + 2);
+        else k.template issue_b<(P + 2) % CYCLE, I, I + 1, MASKED>(s + 2);
     }
 };
 
@@ -320,8 +321,7 @@ struct Kernel {
     int64_t red_len;
     int wave, lane;
     int a_off[4], b_off[4];  // variable parts of the fragment offsets (see fragment_offsets)
-    int active_m;            // 32-row blocks of this wave's 128 tile rows that hold existing rows (wave-uniform)
-    u32x4_t fa[2][MI], fb[2][NI];  // fragments: the block being multiplied and the one being read
+    u32x4_t fa[2][MI], fb[2][NI];  // fragments: the 32-deep block being multiplied and the one being read
 
     template <int P, int I0, int I1, bool MASKED> __device__ __forceinline__ void issue_a(int64_t stage) {
         la.template issue<I0, I1, MASKED>(slab<Pipe::template At<P>::A_SLAB>(), Pipe::template At<P>::A_OFF, stage, red_len);
@@ -331,152 +331,156 @@ struct Kernel {
     }
 
     // Byte offsets of this lane's fragments inside an operand tile.  Only the part that is not a
-    // compile-time constant goes through opaque(): for the K-contiguous layout the tile-row block adds a
-    // constant (32 rows, same swizzle), for the K-strided layout the k16 step does (16 k rows = 8 KiB).
-    template <bool STRIDED, int BLOCKS>
+    // compile-time constant goes through opaque(): for the K-contiguous layout the 16-row block adds a
+    // constant (the swizzle repeats every 16 rows); for the K-strided layout the 32-deep block adds 16 KiB and
+    // the odd 16-column block of a 32-column pair adds 32 bytes (two chunks; the swizzle leaves that bit alone).
+    template <bool STRIDED>
     __device__ __forceinline__ void fragment_offsets(int row0, int (&var)[4]) const {
         if constexpr (STRIDED) {
 #pragma unroll
-            for (int b = 0; b < BLOCKS; ++b) var[b] = opaque(G::kstrided_offset(row0 + b * 32, 0, lane));
+            for (int b = 0; b < 4; ++b) var[b] = opaque(G::kstrided_offset(row0 + b * 32, 0, lane));
         } else {
 #pragma unroll
-            for (int kk = 0; kk < BK / 16; ++kk) var[kk] = opaque(G::kcontig_offset(row0 + (lane & 31), kk, lane >> 5));
+            for (int kb = 0; kb < BK / 32; ++kb) var[kb] = opaque(G::kcontig_offset(row0 + (lane & 15), kb, lane >> 4));
         }
     }
     template <bool STRIDED>
-    __device__ static __forceinline__ int fragment_offset(const int (&var)[4], int block, int kk) {
-        return STRIDED ? var[block] + kk * (16 * BN * 2) : var[kk] + block * (32 * G::ROW_BYTES);
+    __device__ static __forceinline__ int fragment_offset(const int (&var)[4], int block, int kb) {
+        return STRIDED ? var[block >> 1] + (block & 1) * 32 + kb * (32 * BN * 2) : var[kb] + block * (16 * G::ROW_BYTES);
     }
     __device__ __forceinline__ void init_fragments() {
-        fragment_offsets<A_STRIDED, MI>((wave / WAVES_N) * WM, a_off);
-        fragment_offsets<B_STRIDED, NI>((wave % WAVES_N) * WN, b_off);
+        fragment_offsets<A_STRIDED>((wave / WAVES_N) * WM, a_off);
+        fragment_offsets<B_STRIDED>((wave % WAVES_N) * WN, b_off);
     }
 
-    // Fragments of reduction block kk of the stage held at cycle position P.  FULL = false: a tile whose last
-    // rows do not exist (the tail of an expert's rows) only touches this wave's first active_m 32-row blocks.
-    template <int P, bool FULL>
-    __device__ __forceinline__ void read_fragments(int kk, u32x4_t (&af)[MI], u32x4_t (&bf)[NI]) const {
+    // One fragment of the 32-deep block kb of the stage held at ring position P: A block mi / B block ni.
+    template <int P>
+    __device__ __forceinline__ u32x4_t read_a(int kb, int mi) const {
         using At = typename Pipe::template At<P>;
-        const char* ta = slab<At::A_SLAB>();
-        const char* tb = slab<At::B_SLAB>();
+        return read_fragment<A_STRIDED>(slab<At::A_SLAB>(), At::A_OFF + fragment_offset<A_STRIDED>(a_off, mi, kb));
+    }
+    template <int P>
+    __device__ __forceinline__ u32x4_t read_b(int kb, int ni) const {
+        using At = typename Pipe::template At<P>;
+        return read_fragment<B_STRIDED>(slab<At::B_SLAB>(), At::B_OFF + fragment_offset<B_STRIDED>(b_off, ni, kb));
+    }
+    // All fragments of a block.
+    template <int P>
+    __device__ __forceinline__ void read_fragments(int kb, u32x4_t (&af)[MI], u32x4_t (&bf)[NI]) const {
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-            if (FULL || mi < active_m)
-                af[mi] = read_fragment<A_STRIDED>(ta, At::A_OFF + fragment_offset<A_STRIDED>(a_off, mi, kk));
+        for (int ni = 0; ni < NI; ++ni) bf[ni] = read_b<P>(kb, ni);
 #pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-            bf[ni] = read_fragment<B_STRIDED>(tb, At::B_OFF + fragment_offset<B_STRIDED>(b_off, ni, kk));
+        for (int mi = 0; mi < MI; ++mi) af[mi] = read_a<P>(kb, mi);
     }
 
-    template <bool FULL>
-    __device__ __forceinline__ void multiply(const u32x4_t (&af)[MI], const u32x4_t (&bf)[NI], f32x16_t (&acc)[MI][NI]) {
+    // One phase = one 32-deep block = MI * NI matrix instructions of 16 cycles.  A wave that is alone on its SIMD
+    // has nobody to hide its stalls, so the three instruction streams are interleaved by hand: the phase is cut into
+    // 16 slots of four matrix instructions (one A block against half of the B blocks); every slot also reads its share
+    // of the NEXT block's fragments (in the order the next phase needs them: all B blocks within the first slots, then
+    // the A blocks) and every other slot issues one DMA load.  The matrix instructions are inline assembly, which the
+    // instruction scheduler cannot classify, so the order is pinned with a scheduling fence after each slot.
+    // RP / RKB: ring position and block of the fragments being read; LP / LPH: the step and phase whose loads go out.
+    //
+    // The tail tile of an expert's rows runs exactly the same instruction stream on zeros for the rows that do not
+    // exist.  Skipping the missing 16-row blocks was measured and is a LOSS: the 32 work-groups an XCD runs at a
+    // time share their operand panels through the L2 only while they walk the reduction in step; a tile that
+    // finishes early puts its compute unit out of step for the rest of the launch, its requests stop hitting lines
+    // its neighbours brought in, and the launch, which is bound by what the L2 has to fetch, gets 13-16 % slower
+    // (8 tail tiles among 67 at the benchmark shape).
+    template <int RP, int LP, int LPH, bool MASKED>
+    __device__ __forceinline__ void phase(int rkb, int cur, int64_t s, f32x4_t (&acc)[MI][NI]) {
+        constexpr int SLOTS = 2 * MI;  // 16
+        const int nxt = cur ^ 1;
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-            if (FULL || mi < active_m) {
+        for (int slot = 0; slot < SLOTS; ++slot) {
+            const int mi = slot / 2, n0 = (slot & 1) * (NI / 2);
 #pragma unroll
-                for (int ni = 0; ni < NI; ++ni) Mma<T>::run(bf[ni], af[mi], acc[mi][ni]);
+            for (int j = 0; j < NI / 2; ++j) Mma16<T>::run(fb[cur][n0 + j], fa[cur][mi], acc[mi][n0 + j]);
+            // next block's fragments: slots 0-3 read two B blocks each, slots 4-11 one A block each
+            if (slot < 4) {
+                fb[nxt][2 * slot] = read_b<RP>(rkb, 2 * slot);
+                fb[nxt][2 * slot + 1] = read_b<RP>(rkb, 2 * slot + 1);
+            } else if (slot < 4 + MI) {
+                fa[nxt][slot - 4] = read_a<RP>(rkb, slot - 4);
             }
-    }
-
-    // Asks the instruction scheduler to spread the LDS reads (and, with DMA, the loads) of one phase evenly
-    // between its MI*NI matrix instructions, so that a wave that is alone on its SIMD keeps the matrix
-    // pipe busy while its next fragments arrive.
-    template <int I = 0>
-    __device__ static __forceinline__ void interleave_phase() {
-        constexpr int MFMAS = MI * NI;
-        constexpr int READS = (A_STRIDED ? 2 : 1) * MI + (B_STRIDED ? 2 : 1) * NI;
-        constexpr int LOADS = Pipe::PHASE_LOADS;
-        constexpr int SLOTS = 8, READ_SLOTS = 6;  // the last slots of a phase issue no LDS read
-        static_assert(MFMAS % SLOTS == 0, "slots");
-        if constexpr (I < SLOTS) {
-            constexpr int R0 = I < READ_SLOTS ? (READS * I) / READ_SLOTS : READS;
-            constexpr int R1 = I + 1 < READ_SLOTS ? (READS * (I + 1)) / READ_SLOTS : READS;
-            __builtin_amdgcn_sched_group_barrier(0x008, MFMAS / SLOTS, 0);
-            if constexpr (R1 > R0) __builtin_amdgcn_sched_group_barrier(0x100, R1 - R0, 0);
-            constexpr int G = (LOADS * (I + 1)) / SLOTS - (LOADS * I) / SLOTS;
-            if constexpr (G > 0) __builtin_amdgcn_sched_group_barrier(0x020, G, 0);
-            interleave_phase<I + 1>();
+            if (slot % 2 == 1) issue_slot<LP, LPH, MASKED>(slot / 2, s);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
-
-    // One pipeline step at cycle position P on stage s.  On entry the fragments of the stage's first
-    // reduction block are in registers.  Every phase multiplies one block while the next block's fragments
-    // are read and a share of the loads is issued.  Before the last phase the step waits until its own LDS
-    // reads are done and the loads of stage s+1 have landed, and meets the other waves: stage s+1 is then
-    // complete for everybody and nobody reads stage s any more, so its slabs can be refilled while the last
-    // block is multiplied from registers and the first fragments of stage s+1 are read.  A step is
-    // branch-free: stages past the end of the reduction fetch the zero page, which keeps the count of loads
-    // in flight the same at every step and lets the compiler see that the loop needs no other wait on
-    // vector memory.
-    template <int P, int PH, bool FULL, bool MASKED>
-    __device__ __forceinline__ void phases_before_barrier(int64_t s, f32x16_t (&acc)[MI][NI]) {
-        if constexpr (PH + 1 < Pipe::KK) {
-            Pipe::template issue_phase<P, PH, MASKED>(*this, s);
-            read_fragments<P, FULL>(PH + 1, fa[(PH + 1) & 1], fb[(PH + 1) & 1]);
-            multiply<FULL>(fa[PH & 1], fb[PH & 1], acc);
-            if constexpr (FULL) interleave_phase();
-            phases_before_barrier<P, PH + 1, FULL, MASKED>(s, acc);
+    template <int LP, int LPH, bool MASKED>
+    __device__ __forceinline__ void issue_slot(int i, int64_t s) {
+        // i is a constant after unrolling; the loads of a phase are numbered 0 .. PHASE_LOADS - 1
+        switch (i) {
+            case 0: Pipe::template issue_one<LP, LPH, 0, MASKED>(*this, s); break;
+            case 1: Pipe::template issue_one<LP, LPH, 1, MASKED>(*this, s); break;
+            case 2: Pipe::template issue_one<LP, LPH, 2, MASKED>(*this, s); break;
+            case 3: Pipe::template issue_one<LP, LPH, 3, MASKED>(*this, s); break;
+            case 4: Pipe::template issue_one<LP, LPH, 4, MASKED>(*this, s); break;
+            case 5: Pipe::template issue_one<LP, LPH, 5, MASKED>(*this, s); break;
+            case 6: Pipe::template issue_one<LP, LPH, 6, MASKED>(*this, s); break;
+            default: Pipe::template issue_one<LP, LPH, 7, MASKED>(*this, s); break;
         }
     }
-    template <int P, bool FULL, bool MASKED>
-    __device__ __forceinline__ void step(int64_t s, f32x16_t (&acc)[MI][NI]) {
-        constexpr int KK = Pipe::KK;
-        phases_before_barrier<P, 0, FULL, MASKED>(s, acc);
+    // One pipeline step at ring position P on stage s.  On entry the fragments of the stage's first block are in
+    // registers (set 0).  Phase 0 multiplies block 0 while block 1 is read and the A tile of stage s+2 is requested.
+    // Then the step waits until its own LDS reads are done and the loads of stage s+1 have landed, and meets the
+    // other waves: stage s+1 is then complete for everybody and nobody reads stage s any more, so its slabs can be
+    // refilled while block 1 is multiplied from registers and the first fragments of stage s+1 are read.  A step is
+    // branch-free: stages past the end of the reduction fetch the zero page, which keeps the count of loads in
+    // flight the same at every step and lets the compiler see that the loop needs no other wait on vector memory.
+    template <int P, bool MASKED>
+    __device__ __forceinline__ void step(int64_t s, f32x4_t (&acc)[MI][NI]) {
+        static_assert(Pipe::KK == 2 && Pipe::PHASE_LOADS == 8, "two phases of eight loads");
+        phase<P, P, 0, MASKED>(1, 0, s, acc);
         wait_vmcnt_and_lds<Pipe::WAIT>();
         block_barrier();
-        Pipe::template issue_phase<P, KK - 1, MASKED>(*this, s);
-        read_fragments<(P + 1) % Pipe::CYCLE, FULL>(0, fa[KK & 1], fb[KK & 1]);
-        multiply<FULL>(fa[(KK - 1) & 1], fb[(KK - 1) & 1], acc);
-        if constexpr (FULL) interleave_phase();
+        phase<(P + 1) % Pipe::CYCLE, P, 1, MASKED>(0, 1, s, acc);
     }
 
-    template <int P, bool FULL>
-    __device__ __forceinline__ void steps_from(int64_t s, int64_t count, f32x16_t (&acc)[MI][NI]) {
+    template <int P>
+    __device__ __forceinline__ void steps_from(int64_t s, int64_t count, f32x4_t (&acc)[MI][NI]) {
         if constexpr (P < Pipe::CYCLE) {
             if (P < count) {
-                step<P, FULL, true>(s + P, acc);
-                steps_from<P + 1, FULL>(s, count, acc);
+                step<P, true>(s + P, acc);
+                steps_from<P + 1>(s, count, acc);
             }
         }
     }
-    template <int P, bool FULL, bool MASKED>
-    __device__ __forceinline__ void full_cycle(int64_t s, f32x16_t (&acc)[MI][NI]) {
+    template <int P, bool MASKED>
+    __device__ __forceinline__ void full_cycle(int64_t s, f32x4_t (&acc)[MI][NI]) {
         if constexpr (P < Pipe::CYCLE) {
-            step<P, FULL, MASKED>(s + P, acc);
-            full_cycle<P + 1, FULL, MASKED>(s, acc);
+            step<P, MASKED>(s + P, acc);
+            full_cycle<P + 1, MASKED>(s, acc);
         }
     }
 
     // `plain_steps`: the first that many steps only issue loads of stages that lie wholly inside the reduction, in a
     // tile without missing rows or columns; they take the unmasked form of the loads.
-    template <bool FULL>
-    __device__ __forceinline__ void run_stages(int64_t num_stages, int64_t plain_steps, f32x16_t (&acc)[MI][NI]) {
-        read_fragments<0, FULL>(0, fa[0], fb[0]);
+    __device__ __forceinline__ void run_stages(int64_t num_stages, int64_t plain_steps, f32x4_t (&acc)[MI][NI]) {
+        read_fragments<0>(0, fa[0], fb[0]);
         int64_t s = 0;
-        if constexpr (FULL)
-            for (; s + Pipe::CYCLE <= plain_steps; s += Pipe::CYCLE) full_cycle<0, FULL, false>(s, acc);
-        for (; s + Pipe::CYCLE <= num_stages; s += Pipe::CYCLE) full_cycle<0, FULL, true>(s, acc);
-        steps_from<0, FULL>(s, num_stages - s, acc);  // fewer than CYCLE steps remain
+        for (; s + Pipe::CYCLE <= plain_steps; s += Pipe::CYCLE) full_cycle<0, false>(s, acc);
+        for (; s + Pipe::CYCLE <= num_stages; s += Pipe::CYCLE) full_cycle<0, true>(s, acc);
+        steps_from<0>(s, num_stages - s, acc);  // fewer than CYCLE steps remain
     }
 
-    __device__ __forceinline__ void run(f32x16_t (&acc)[MI][NI]) {
+    __device__ __forceinline__ void run(f32x4_t (&acc)[MI][NI]) {
         const int64_t num_stages = (red_len + BK - 1) / BK;
         if (num_stages > 0) {
             Pipe::prologue(*this);
             wait_vmcnt<Pipe::PROLOGUE_WAIT>();
             block_barrier();
-            // The two loops issue the same loads and meet at the same barriers, so waves of one work-group may
-            // take different ones.  The row-grouped kinds take the second for the tail tile of an expert's rows:
-            // its cost then follows the rows that exist (plus the full weight panel it still has to stream).
-            if (KIND == XMA_GEMM_MT || active_m == MI) {
-                // wave-uniform: validity is a property of rows and columns of the tile, combined over the lanes
-                const bool whole = __builtin_amdgcn_readfirstlane(__all((int)(la.all_valid() && lb.all_valid()))) != 0;
-                const int64_t plain = whole ? red_len / BK - Pipe::LOOKAHEAD : 0;
-                run_stages<true>(num_stages, plain, acc);
-            } else {
-                run_stages<false>(num_stages, 0, acc);
-            }
+            // wave-uniform: validity is a property of rows and columns of the tile, combined over the lanes; the
+            // plain and the masked loops issue the same loads and meet at the same barriers, so the waves of a
+            // work-group may disagree
+            const bool whole = __builtin_amdgcn_readfirstlane(__all((int)(la.all_valid() && lb.all_valid()))) != 0;
+            const int64_t plain = whole ? red_len / BK - Pipe::LOOKAHEAD : 0;
+            run_stages(num_stages, plain, acc);
             wait_vmcnt<0>();  // the trailing zero-page loads
+            // The matrix instructions are inline assembly, so the compiler does not know that the accumulators are
+            // still being written when the loop ends and would not keep the distance the hardware needs between a
+            // matrix instruction and a read of its result: 32 idle cycles cover it.
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         }
         block_barrier();  // every wave is done reading the slabs; no load is in flight any more
     }
@@ -584,20 +588,11 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         }
     }
     k.init_fragments();
-    k.active_m = MI;
-    if constexpr (KIND != XMA_GEMM_MT) {
-        const int rows_here = (int)(m_end - m_begin) - (k.wave / WAVES_N) * WM;
-        const int blocks = (rows_here + 31) / 32;
-        k.active_m = __builtin_amdgcn_readfirstlane(blocks < 0 ? 0 : blocks > MI ? MI : blocks);
-    }
-
-    f32x16_t acc[MI][NI];
+    f32x4_t acc[MI][NI];
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
+        for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     k.run(acc);
 
@@ -633,9 +628,9 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-                    for (int g = 0; g < 8; ++g) {
+                    for (int g = 0; g < 2; ++g) {
                         const float2 v{acc[mi][ni][2 * g], acc[mi][ni][2 * g + 1]};
-                        __hip_atomic_store(mine + ((mi * NI + ni) * 8 + g) * THREADS + tid, __builtin_bit_cast(uint64_t, v),
+                        __hip_atomic_store(mine + ((mi * NI + ni) * 2 + g) * THREADS + tid, __builtin_bit_cast(uint64_t, v),
                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
             wait_vmcnt<0>();  // this wave's partial sums have reached memory ...
@@ -651,35 +646,39 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-                for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
+                for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
             // The sums are requested 32 loads at a time and added afterwards: with all 256 accumulators live the
             // compiler otherwise fetches them one by one, a full memory latency each.
             for (int part = 0; part < work.parts; ++part) {
                 const uint64_t* src = part_buffer(part);
 #pragma unroll
-                for (int mi = 0; mi < MI; ++mi) {
-                    uint64_t v[NI][8];
+                for (int m2 = 0; m2 < MI / 2; ++m2) {
+                    uint64_t v[2][NI][2];
 #pragma unroll
-                    for (int ni = 0; ni < NI; ++ni)
+                    for (int h = 0; h < 2; ++h)
 #pragma unroll
-                        for (int g = 0; g < 8; ++g)
-                            v[ni][g] = __hip_atomic_load(src + ((mi * NI + ni) * 8 + g) * THREADS + tid, __ATOMIC_RELAXED,
-                                                         __HIP_MEMORY_SCOPE_AGENT);
+                        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                            for (int g = 0; g < 2; ++g)
+                                v[h][ni][g] = __hip_atomic_load(src + (((2 * m2 + h) * NI + ni) * 2 + g) * THREADS + tid,
+                                                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     batch_fence();
 #pragma unroll
-                    for (int ni = 0; ni < NI; ++ni)
+                    for (int h = 0; h < 2; ++h)
 #pragma unroll
-                        for (int g = 0; g < 8; ++g) pin(v[ni][g]);
+                        for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-                    for (int ni = 0; ni < NI; ++ni)
+                            for (int g = 0; g < 2; ++g) pin(v[h][ni][g]);
 #pragma unroll
-                        for (int g = 0; g < 8; ++g) {
-                            const float2 f = __builtin_bit_cast(float2, v[ni][g]);
-                            acc[mi][ni][2 * g] += f.x;
-                            acc[mi][ni][2 * g + 1] += f.y;
-                        }
+                    for (int h = 0; h < 2; ++h)
+#pragma unroll
+                        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                            for (int g = 0; g < 2; ++g) {
+                                const float2 f = __builtin_bit_cast(float2, v[h][ni][g]);
+                                acc[2 * m2 + h][ni][2 * g] += f.x;
+                                acc[2 * m2 + h][ni][2 * g + 1] += f.y;
+                            }
                     batch_fence();
                 }
             }
@@ -717,11 +716,11 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
         return (uint32_t)(r < rows_here ? r : rows_here - 1);
     };
 
-    int32_t orow[MI][IT];  // output row of each owned row (of the last existing row for rows past the end)
+    int32_t orow[OUT_SLABS][IT];  // output row of each owned row (of the last existing row for rows past the end)
     if constexpr (KIND != XMA_GEMM_MT) {
         auto fill = [&](auto index_of) {
 #pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
+            for (int mi = 0; mi < OUT_SLABS; ++mi)
 #pragma unroll
                 for (int it = 0; it < IT; ++it) orow[mi][it] = index_of(safe_row(mi, it));
             batch_fence();  // the loads stay in flight while the accumulators are packed; they are waited for after that
@@ -756,67 +755,70 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     };
     if constexpr (SWBWD) load_saved(0, hu[0], hg[0]);
 
-    // MFMA result element r of lane l: tile column 8*(r/4) + 4*(l/32) + r%4 (+32*ni), tile row l%32 (+32*mi).
-    // A 512-byte LDS row holds 32 chunks of 8 columns; chunk c of buffer row br sits at c ^ (br & 31).
+    // MFMA result register r of lane l in block (mi, ni): tile row 16*mi + l%16, tile column 16*ni + 4*(l/16) + r.
+    // Slab s holds the tile rows {wr*128 + s*32 + 0..31} of both wave rows as buffer rows wr*32 + 0..31, i.e. the
+    // blocks mi = 2s and 2s+1.  A 512-byte LDS row holds 32 chunks of 8 columns; chunk c of buffer row br sits at
+    // c ^ (br & 31).
     {
         const int wn0 = (k.wave % WAVES_N) * WN;
-        const int br = (k.wave / WAVES_N) * 32 + (etid & 31);
-        const int half = (etid >> 5) & 1;
+        const int br0 = (k.wave / WAVES_N) * 32 + (etid & 15);  // buffer row of the even block of a slab
+        const int quarter = (etid >> 4) & 3;
         // Forward kinds: the expert's bias row, added to the fp32 sums before they are rounded.  Tile column c is
         // weight row n0 + c, or for a gated tile n0 + c (c < 128) and N/2 + n0 + c - 128 (c >= 128).
-        float bias[KIND == XMA_GEMM_TN ? NI : 1][KIND == XMA_GEMM_TN ? 4 : 1][KIND == XMA_GEMM_TN ? 4 : 1];
+        float bias[KIND == XMA_GEMM_TN ? NI : 1][KIND == XMA_GEMM_TN ? 4 : 1];
         bool with_bias = false;
         if constexpr (KIND == XMA_GEMM_TN) {
             with_bias = P.bias != nullptr;
             if (with_bias) {
                 const T* row = reinterpret_cast<const T*>(P.bias) + (int64_t)expert * P.ld_bias;
 #pragma unroll
-                for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int c = wn0 + ni * 32 + 8 * g + 4 * half;
-                        int64_t n;
-                        bool exists;
-                        if constexpr (EPI == EPI_PAIRED) {
-                            const int64_t half_n = P.n / 2;
-                            n = n0 + (c % BN_OUT) + (c >= BN_OUT ? half_n : 0);
-                            exists = n0 + (c % BN_OUT) < half_n;
-                        } else {
-                            n = n0 + c;
-                            exists = n < P.n;
-                        }
-                        const uint2 raw = *reinterpret_cast<const uint2*>(row + (exists ? n : 0));
-                        float v[8];
-                        Elem<T>::unpack(make_uint4(raw.x, raw.y, 0u, 0u), v);
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) bias[ni][g][q] = exists ? v[q] : 0.0f;
+                for (int ni = 0; ni < NI; ++ni) {
+                    const int c = wn0 + ni * 16 + 4 * quarter;
+                    int64_t n;
+                    bool exists;
+                    if constexpr (EPI == EPI_PAIRED) {
+                        const int64_t half_n = P.n / 2;
+                        n = n0 + (c % BN_OUT) + (c >= BN_OUT ? half_n : 0);
+                        exists = n0 + (c % BN_OUT) < half_n;
+                    } else {
+                        n = n0 + c;
+                        exists = n < P.n;
                     }
+                    const uint2 raw = *reinterpret_cast<const uint2*>(row + (exists ? n : 0));
+                    float v[8];
+                    Elem<T>::unpack(make_uint4(raw.x, raw.y, 0u, 0u), v);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) bias[ni][q] = exists ? v[q] : 0.0f;
+                }
             }
         }
         // (the bias is a copy of the code of its own: a wave alone on its SIMD pays for every instruction, and as
         // one copy the compiler adds a selected zero to every sum of a launch that has no bias)
-        auto write_rows = [&](char* buf, const f32x16_t (&a)[NI], auto bias_tag) {
+        auto write_rows = [&](char* buf, const f32x4_t (&even)[NI], const f32x4_t (&odd)[NI], auto bias_tag) {
             constexpr bool BIAS = decltype(bias_tag)::value;
 #pragma unroll
-            for (int ni = 0; ni < NI; ++ni) {
+            for (int h = 0; h < 2; ++h) {
+                const int br = br0 + 16 * h;
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int chunk = ((wn0 + ni * 32 + 8 * g) >> 3) ^ (br & 31);
-                    float v[4] = {a[ni][4 * g], a[ni][4 * g + 1], a[ni][4 * g + 2], a[ni][4 * g + 3]};
+                for (int ni = 0; ni < NI; ++ni) {
+                    const f32x4_t& a = h == 0 ? even[ni] : odd[ni];
+                    const int c = wn0 + ni * 16 + 4 * quarter;
+                    const int chunk = (c >> 3) ^ (br & 31);
+                    float v[4] = {a[0], a[1], a[2], a[3]};
                     if constexpr (BIAS) {
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) v[q] += bias[KIND == XMA_GEMM_TN ? ni : 0][KIND == XMA_GEMM_TN ? g : 0][KIND == XMA_GEMM_TN ? q : 0];
+                        for (int q = 0; q < 4; ++q) v[q] += bias[KIND == XMA_GEMM_TN ? ni : 0][KIND == XMA_GEMM_TN ? q : 0];
                     }
-                    *reinterpret_cast<uint2*>(buf + br * (BN * 2) + (chunk << 4) + half * 8) =
+                    *reinterpret_cast<uint2*>(buf + br * (BN * 2) + (chunk << 4) + (quarter & 1) * 8) =
                         make_uint2(Elem<T>::pack2(v[0], v[1]), Elem<T>::pack2(v[2], v[3]));
                 }
             }
         };
         auto write_all = [&](auto bias_tag) {
-            write_rows(slab<0>(), acc[0], bias_tag);
-            write_rows(slab<1>(), acc[1], bias_tag);
-            write_rows(slab<2>(), acc[2], bias_tag);
-            write_rows(slab<3>(), acc[3], bias_tag);
+            write_rows(slab<0>(), acc[0], acc[1], bias_tag);
+            write_rows(slab<1>(), acc[2], acc[3], bias_tag);
+            write_rows(slab<2>(), acc[4], acc[5], bias_tag);
+            write_rows(slab<3>(), acc[6], acc[7], bias_tag);
         };
         if (KIND == XMA_GEMM_TN && with_bias) write_all(std::true_type{});
         else write_all(std::false_type{});
@@ -824,7 +826,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
     if constexpr (KIND != XMA_GEMM_MT) {
         batch_fence();
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
+        for (int mi = 0; mi < OUT_SLABS; ++mi)
 #pragma unroll
             for (int it = 0; it < IT; ++it) pin(orow[mi][it]);
     }
@@ -928,7 +930,7 @@ __global__ __launch_bounds__(THREADS) void grouped_gemm_dma_kernel(const GemmPar
             else rows(std::integral_constant<int, ACT_GLU>{});
         } else {  // EPI_BACKWARD
             const int64_t n = n0 + cc * PV;
-            if constexpr (mi + 1 < MI) load_saved(mi + 1, hu[(mi + 1) & 1], hg[(mi + 1) & 1]);
+            if constexpr (mi + 1 < OUT_SLABS) load_saved(mi + 1, hu[(mi + 1) & 1], hg[(mi + 1) & 1]);
             u32x4_t dv[IT];
             read_own_chunks(dv);
             auto rows = [&](auto act_tag) {
