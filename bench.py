@@ -119,6 +119,9 @@ def _parse() -> argparse.Namespace:
                     help="run only that one of the other configurations (the command its profile is taken with)")
     ap.add_argument("--library-gemm-only", action="store_true",
                     help="run only the loop of library GEMMs (the command the library's counter profile is taken with)")
+    ap.add_argument("--reduction-sweep", action="store_true",
+                    help="run only the sweep over the reduction length that separates a tile's fixed cost from its "
+                    "cost per reduction step, for the grouped kernel and for the library's dense GEMM")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument(
         "--copy-probe",
@@ -389,6 +392,59 @@ def _library_gemms(T: int, H: int, I: int, E: int, k: int, iters: int = 3) -> di
     }
 
 
+def _reduction_sweep(M: int = 16384, N: int = 16384, E: int = 8, iters: int = 8) -> dict:
+    """[M, K] x [N, K]^T in bf16 with M / E rows per expert (no ragged tiles, identity row map) for a range of
+    reduction lengths K, with the grouped kernel and with one dense library GEMM of the same size.  M x N is a whole
+    number of rounds of 256 tiles of 256 x 256, so the time of a round is a straight line in K: its slope is what
+    the main loop costs, its intercept what a tile costs outside the loop (finding the tile, first loads, epilogue,
+    the hand-over to the next work-group)."""
+
+    import numpy as np
+    import torch
+
+    from flash_model_architectures_amd import ops
+
+    dev, dt = "cuda", torch.bfloat16
+    rounds = (M // 256) * (N // 256) / 256.0
+    offsets = torch.arange(0, M + 1, M // E, dtype=torch.int32, device=dev)
+    rows = torch.arange(M, dtype=torch.int32, device=dev)
+    expert_of_row = torch.repeat_interleave(torch.arange(E, device=dev), M // E).int()
+    out = torch.empty(M, N, device=dev, dtype=dt)
+
+    def timed(fn) -> float:
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / iters * 1e3  # microseconds
+
+    points = []
+    for K in (1024, 2048, 4096, 8192, 14336):
+        a = torch.randn(M, K, device=dev).to(dt)
+        w = (torch.randn(E, N, K, device=dev) * 0.02).to(dt)
+        ours = timed(lambda: ops.scatter2scatter(a, w.permute(0, 2, 1), expert_of_row, rows, out, 1, True, True, offsets))
+        dense = timed(lambda: torch.matmul(a, w[0].t(), out=out))
+        flops = 2.0 * M * N * K
+        points.append({"K": K, "grouped_us_per_round": round(ours / rounds, 2), "library_us_per_round": round(dense / rounds, 2),
+                       "grouped_frac_of_bf16_peak": round(flops / (ours * 1e-6) / PEAK_BF16_FLOPS, 4),
+                       "library_frac_of_bf16_peak": round(flops / (dense * 1e-6) / PEAK_BF16_FLOPS, 4)})
+        del a, w
+    ks = np.array([p["K"] for p in points], dtype=np.float64)
+    fit = {}
+    for who in ("grouped", "library"):
+        slope, intercept = np.polyfit(ks, np.array([p[f"{who}_us_per_round"] for p in points]), 1)
+        fit[who] = {"us_per_round_outside_the_loop": round(float(intercept), 2),
+                    "us_per_round_per_1024_of_reduction": round(float(slope) * 1024, 2),
+                    "frac_of_bf16_peak_of_the_loop_alone": round(2.0 * 256 * 256 * 256 * 1024 / (slope * 1024 * 1e-6) / PEAK_BF16_FLOPS, 4)}
+    return {"what": f"[{M}, K] x [{N}, K]^T, bf16, {E} experts of {M // E} rows, {rounds:g} rounds of 256 tiles; "
+                    "least-squares line through the times per round", "points": points, "fit": fit}
+
+
 def _aux_hbm_kernels(T: int, H: int, I: int, E: int, k: int) -> list:
     """Stand-alone timings (events on the current stream, outside the timed steps) of the HBM-bound kernels of
     the path at this workload's sizes, plus the histogram / permutation / row moves at fixed large sizes
@@ -470,6 +526,9 @@ def main() -> int:
     if args.only_config is not None:
         workload = OTHER_WORKLOADS[0 if args.only_config == "fine-grained" else 1]
         print(json.dumps({"other_configs": [_other_config(workload, args.other_steps, 2)]}))
+        return 0
+    if args.reduction_sweep:
+        print(json.dumps({"reduction_sweep": _reduction_sweep()}))
         return 0
     if args.library_gemm_only:
         print(json.dumps({"library_gemm": _library_gemms(T, H, I, E, k, iters=max(args.steps, 1))}))

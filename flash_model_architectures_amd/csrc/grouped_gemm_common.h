@@ -13,10 +13,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // 16 bytes moved as ONE vector access
 
 constexpr int kNumXcd = 8;     // accelerator complex dies, each with a private L2
-#ifndef XMA_BAND_TILES
-#define XMA_BAND_TILES 4
-#endif
-constexpr int kBandTiles = XMA_BAND_TILES;  // row tiles per band of the tile walk
+constexpr int kBandTiles = 4;  // row tiles per band of the tile walk (2, 8 and 16 measured slower)
 
 // ---- kernel arguments -----------------------------------------------------------------------------
 struct GemmParams {
