@@ -124,7 +124,7 @@ def test_all_layouts_and_epilogues(case, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("activation", ["swiglu", "glu", "gelu_tanh"])
-@pytest.mark.parametrize("case", [CASES[0], CASES[3], CASES[4]])
+@pytest.mark.parametrize("case", [CASES[0], CASES[3], CASES[4], CASES[6], CASES[7]])
 def test_fused_activations_and_bias(case, activation, dtype):
     """Every activation the epilogues fuse, forward and backward, with and without the per-expert bias that the
     forward kernels add to the fp32 product: against the torch modules the reference's test drives the layer with
