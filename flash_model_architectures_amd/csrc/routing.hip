@@ -147,10 +147,7 @@ __device__ __forceinline__ void place_batch(int64_t e64, int64_t i, int E, int n
     }
     uint32_t base = 0;
     const int leader = ok ? (int)__ffsll((unsigned long long)peers) - 1 : lane;
-    if (ok && leader == lane) {
-        base = next[e];
-        next[e] = base + (uint32_t)__popcll(peers);
-    }
+    if (ok && leader == lane) base = atomicAdd(&next[e], (uint32_t)__popcll(peers));  // one LDS round trip, not two
     base = __shfl(base, leader, kWaveSize);
     if (ok) {
         const uint32_t pos = base + (uint32_t)__popcll(peers & (((uint64_t)1 << lane) - 1));
@@ -166,14 +163,14 @@ __global__ __launch_bounds__(256) void unit_hist_kernel(const IdT* __restrict__ 
     const int wave = threadIdx.x / kWaveSize;
     const int lane = lane_id();
     uint32_t* mine = lds_hist + wave * E;
-    for (int i = lane; i < E; i += kWaveSize) mine[i] = 0;
-    __syncthreads();
     const int64_t unit = (int64_t)blockIdx.x * waves_per_block + wave;
     const int64_t begin = unit * kChunk;
+    const int64_t end = begin + kChunk < n ? begin + kChunk : n;
+    int64_t v[kBatches];
+    load_chunk(ids, begin < n ? begin : n, end, lane, v);  // requested before the LDS row is cleared (all -1 past n)
+    for (int i = lane; i < E; i += kWaveSize) mine[i] = 0;
+    __syncthreads();
     if (begin < n) {
-        const int64_t end = begin + kChunk < n ? begin + kChunk : n;
-        int64_t v[kBatches];
-        load_chunk(ids, begin, end, lane, v);
 #pragma unroll
         for (int j = 0; j < kBatches; ++j)
             if (v[j] >= 0 && v[j] < E) atomicAdd(&mine[v[j]], 1u);
@@ -335,6 +332,11 @@ __global__ __launch_bounds__(256) void scan_place_kernel(const IdT* __restrict__
     const int64_t end = begin + kChunk < n ? begin + kChunk : n;
     int64_t v[kBatches];
     load_chunk(ids, begin, end, lane, v);  // all -1 for a unit past the end
+    // ... and so are the histograms of the block's own units (thread e: expert e), which are needed after the scan
+    uint32_t own[kFusedUnitsPerBlock];
+#pragma unroll
+    for (int w = 0; w < kFusedUnitsPerBlock; ++w)
+        own[w] = (int)threadIdx.x < E && first_unit + w < units ? unit_hist[(first_unit + w) * E + threadIdx.x] : 0u;
 
     for (int i = threadIdx.x; i < 2 * E; i += 256) lds_hist[i] = 0;
     __syncthreads();
@@ -390,10 +392,6 @@ __global__ __launch_bounds__(256) void scan_place_kernel(const IdT* __restrict__
             if (e == E - 1) offsets[E] = (int32_t)(first_slot + count);
         }
         // first output slot of the ids of expert e in each of the block's units
-        uint32_t own[kFusedUnitsPerBlock];
-#pragma unroll
-        for (int w = 0; w < kFusedUnitsPerBlock; ++w)
-            own[w] = first_unit + w < units ? unit_hist[(first_unit + w) * E + e] : 0u;
         uint32_t slot = first_slot + before[e];
 #pragma unroll
         for (int w = 0; w < kFusedUnitsPerBlock; ++w) {
