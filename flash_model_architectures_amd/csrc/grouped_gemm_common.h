@@ -257,7 +257,7 @@ inline int64_t grid_for_tiles(int64_t row_tiles, int64_t col_tiles) {
 
 inline int64_t max_row_tiles(int64_t rows, int E, int BM) { return rows / BM + E; }
 
-// The MFMA instruction the 16-bit kernels are built on: acc(32x32) += X(32 x 16) * Y(32 x 16)^T,
+// The MFMA instruction of the register-staged kernel for 16-bit types: acc(32x32) += X(32 x 16) * Y(32 x 16)^T,
 // lane l supplies row l%32 and the 8 reduction elements 8*(l/32)..8*(l/32)+7 of both operands.
 template <typename T>
 struct Mma;
@@ -269,7 +269,7 @@ struct Mma<bf16_t> {
                                                       acc, 0, 0, 0);
     }
 };
-// The 16x16x32 form: acc(16x16) += X(16 x 32) * Y(16 x 32)^T; lane l supplies row l%16 and the 8 reduction
+// The 16x16x32 form, which the LDS-DMA kernel is built on: acc(16x16) += X(16 x 32) * Y(16 x 32)^T; lane l supplies row l%16 and the 8 reduction
 // elements 8*(l/16)..+7 of both operands; result register r of lane l is D[4*(l/16) + r][l%16] (rows from X).  Half the
 // accumulator traffic per FLOP of the 32x32x16 form: under the device's power cap it sustains a higher clock.  Written
 // as inline assembly with the accumulator tied in place: the compiler's builtin has no tied form for a four-register

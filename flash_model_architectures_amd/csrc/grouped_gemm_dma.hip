@@ -5,14 +5,16 @@
 // itself (ds_read_b64_tr_b16).
 //
 // Tile 256 x 256 per work-group, 4 waves as 2 x 2, one wave per SIMD with the whole 512-register budget:
-// each wave owns 128 x 128 (4 x 4 MFMA 32x32x16 tiles, 256 accumulator registers).  A wave that is alone
-// on its SIMD has nobody to hide its stalls, so the main loop is software-pipelined by hand: the fragments
-// of reduction block k+1 are read from LDS while block k is multiplied, DMA loads are dealt out a few per
-// block, and the instruction scheduler is told how to interleave the three streams.
+// each wave owns 128 x 128 (8 x 8 blocks of the 16x16x32 matrix instruction, 256 accumulator registers).  A
+// wave that is alone on its SIMD has nobody to hide its stalls, so the main loop is software-pipelined by hand:
+// the fragments of the 32-deep reduction block k+1 are read from LDS while block k is multiplied, DMA loads are
+// dealt out one every eight matrix instructions, and the order of the three streams is pinned slot by slot.
 //
-// What bounds the loop (measured): a compute unit pulls a 256 x 256 tile's operands from L2 at
-// 128 FLOP per byte, and the L2 delivers whole 128-byte lines about 1.5 x faster than half lines.  So
-// K-contiguous operands are staged 64 reduction elements at a time (128-byte rows); see Ring64x5.
+// What bounds the loop (measured): what the L2 has to fetch and deliver.  A compute unit pulls a 256 x 256
+// tile's operands from L2 at 128 FLOP per byte, the L2 delivers whole 128-byte lines about 1.5 x faster than
+// half lines (so K-contiguous operands are staged 64 reduction elements at a time, 128-byte rows; see
+// Ring64x5), and the 32 tiles an XCD runs at a time share their operand panels in its L2 as long as they walk
+// the reduction in step (see Kernel::phase).
 //
 // LDS is a pool of five 32 KiB slabs (all 160 KiB of the compute unit).
 // Tile layouts inside a slab:
@@ -276,7 +278,7 @@ struct OperandLoads {
 
 // ---- pipeline policies --------------------------------------------------------------------------------------
 // A policy says where the tiles of stage j live, which loads the step at cycle position P issues in
-// each of its phases (one phase = 16 reduction elements), and how many loads may still be in flight when
+// each of its phases (one phase = 32 reduction elements), and how many loads may still be in flight when
 // the step reaches its barrier.  Loads are spread evenly over the phases: the texture path of a compute
 // unit takes about sixteen cycles per DMA instruction and a wave that issues into a full queue stalls,
 // matrix instructions included.
