@@ -551,10 +551,11 @@ def _weight_layout(W: torch.Tensor) -> tuple[int, int]:
     """(kind, row stride) of a logical [E, K, N] weight tensor from its strides."""
 
     assert W.dim() == 3
+    # (the stride of a dimension of size 1 means nothing; the row stride handed to the kernel must still cover a row)
     if W.stride(1) == 1 and (W.size(2) == 1 or W.stride(2) >= W.size(1)):
-        return nat.GEMM_TN, W.stride(2)  # stored [E, N, K]
+        return nat.GEMM_TN, W.stride(2) if W.size(2) > 1 else max(W.stride(2), W.size(1))  # stored [E, N, K]
     if W.stride(2) == 1 and (W.size(1) == 1 or W.stride(1) >= W.size(2)):
-        return nat.GEMM_NN, W.stride(1)  # stored [E, K, N]
+        return nat.GEMM_NN, W.stride(1) if W.size(1) > 1 else max(W.stride(1), W.size(2))  # stored [E, K, N]
     raise ValueError(f"expert weights need one unit stride among the last two dims, got strides {W.stride()}")
 
 
@@ -644,7 +645,10 @@ def group_bwd_W(
         assert x_index.numel() == rows
     else:
         assert X.size(0) == rows
-    if x_index is not None and X.dtype != torch.float32 and DW.stride(1) == 1:
+    # (the stride of a dimension of size 1 means nothing: it neither decides the layout nor serves as a row stride)
+    n_major = DW.stride(1) == 1 and (DW.size(2) == 1 or DW.stride(2) >= DW.size(1))
+    k_major = DW.stride(2) == 1 and (DW.size(1) == 1 or DW.stride(1) >= DW.size(2))
+    if x_index is not None and X.dtype != torch.float32 and n_major:
         # the LDS-DMA kernel walks the routed rows with a fixed stride, so 16-bit activations are
         # gathered once (an HBM-bound pass two orders of magnitude cheaper than the GEMM)
         gathered = torch.empty(rows, X.size(1), dtype=X.dtype, device=X.device)
@@ -660,7 +664,7 @@ def group_bwd_W(
         c_expert_stride=DW.stride(0),
         expert_offsets=expert_offsets,
     )
-    if DW.stride(1) == 1:  # storage [E, N, K]: rows of C[e] come from DY, columns from X
+    if n_major:  # storage [E, N, K]: rows of C[e] come from DY, columns from X
         _grouped_gemm(
             n=DY.size(1),
             k=X.size(1),
@@ -668,12 +672,12 @@ def group_bwd_W(
             lda=_row_stride(DY),
             b=X,
             ldb=_row_stride(X),
-            ldc=DW.stride(2),
+            ldc=DW.stride(2) if DW.size(2) > 1 else max(DW.stride(2), DW.size(1)),
             in_index=x_index,
             in_fan_out=x_fan_out,
             **common,
         )
-    elif DW.stride(2) == 1:  # storage [E, K, N]: rows of C[e] come from X
+    elif k_major:  # storage [E, K, N]: rows of C[e] come from X
         if x_index is not None:
             gathered = torch.empty(rows, X.size(1), dtype=X.dtype, device=X.device)
             group(X, x_index, gathered, None, x_fan_out)
@@ -685,7 +689,7 @@ def group_bwd_W(
             lda=_row_stride(X),
             b=DY,
             ldb=_row_stride(DY),
-            ldc=DW.stride(1),
+            ldc=DW.stride(1) if DW.size(1) > 1 else max(DW.stride(1), DW.size(2)),
             **common,
         )
     else:

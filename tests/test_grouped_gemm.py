@@ -36,6 +36,8 @@ CASES = [
     (513, 200, 104, 5, 3, (4,)),
     (300, 100, 52, 4, 2, ()),  # neither H nor I a multiple of the vector width: the element-wise kernel
     (129, 66, 35, 3, 2, (1,)),  # odd I: rows of the activation start at odd elements
+    (50, 1, 24, 3, 2, ()),  # H = 1: torch reports arbitrary strides for a dimension of size 1
+    (40, 24, 1, 2, 1, ()),  # I = 1
 ]
 
 
