@@ -706,6 +706,9 @@ int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
         XMA_REQUIRE(a.epilogue == XMA_EPI_NONE || (a.kind == XMA_GEMM_TN && forward_epi) ||
                         (a.kind == XMA_GEMM_NN && backward_epi),
                     "xma_grouped_gemm: epilogue %d not available for kind %d", a.epilogue, a.kind);
+        // nothing to do, and nothing to hold the views of empty tensors to (their pointers may be null and their
+        // strides anything)
+        if (a.rows == 0 || a.n == 0) return 0;
         XMA_REQUIRE(a.lda >= a.k, "xma_grouped_gemm: lda too small");
         XMA_REQUIRE(a.ldb >= (a.kind == XMA_GEMM_TN ? a.k : a.n), "xma_grouped_gemm: ldb too small");
         if (shape == EPI_PAIRED) {
@@ -725,13 +728,13 @@ int xma_grouped_gemm(const xma_grouped_gemm_args* args, void* stream_) {
         }
         XMA_REQUIRE(a.bias == nullptr || (a.kind == XMA_GEMM_TN && a.ld_bias >= a.n),
                     "xma_grouped_gemm: bias needs a forward (TN) kind and ld_bias >= n");
-        if (a.rows == 0 || a.n == 0) return 0;
         XMA_REQUIRE(a.workspace != nullptr &&
                         a.workspace_bytes >= xma_grouped_gemm_workspace_bytes(a.num_experts, a.rows),
                     "xma_grouped_gemm: workspace too small (%lld < %lld)", (long long)a.workspace_bytes,
                     (long long)xma_grouped_gemm_workspace_bytes(a.num_experts, a.rows));
     }
-    XMA_REQUIRE(a.a && a.b && a.c, "xma_grouped_gemm: null operand");
+    // (without rows the weight-gradient kind still writes its zeros; its operands, which may then be null, are never read)
+    XMA_REQUIRE(a.c && (a.rows == 0 || (a.a && a.b)), "xma_grouped_gemm: null operand");
     hipStream_t stream = (hipStream_t)stream_;
     // a gated tile of the vector kernels pairs whole 16-byte chunks of the two halves
     const bool paired_tail = (a.epilogue == XMA_EPI_SWIGLU || a.epilogue == XMA_EPI_GLU) && a.n % (2 * pv) != 0;

@@ -36,6 +36,8 @@ def _row_stride(t: torch.Tensor) -> int:
     """Row stride of a 2-D tensor whose rows are contiguous."""
 
     assert t.dim() == 2, "expected a 2-D tensor"
+    if t.size(0) == 0:  # no rows: torch calls any strides contiguous (an expanded gradient keeps its zeros)
+        return max(t.size(1), 1)
     assert t.size(1) <= 1 or t.stride(1) == 1, "rows must be contiguous"
     return t.stride(0) if t.size(0) > 1 else max(t.stride(0), t.size(1))
 
@@ -373,8 +375,11 @@ def expert_colsum(src: torch.Tensor, expert_offsets: torch.Tensor, out: torch.Te
     nat.require_device(src, expert_offsets, out)
     E = out.size(0)
     assert src.dim() == 2 and out.dim() == 2 and src.size(1) == out.size(1) and src.dtype == out.dtype
-    assert src.stride(1) == 1 and out.stride(1) == 1
+    assert (src.size(0) == 0 or src.stride(1) == 1) and out.stride(1) == 1
     assert expert_offsets.dtype == torch.int32 and expert_offsets.is_contiguous() and expert_offsets.numel() == E + 1
+    if src.size(0) == 0:  # no rows: every expert's sum is zero (an empty tensor has no memory to hand to the kernel)
+        out.zero_()
+        return
     nat.call(
         "xma_expert_colsum",
         src.data_ptr(),

@@ -330,6 +330,26 @@ def test_skewed_routing_full_size_sampled():
         assert bool(torch.all(grad[torch.as_tensor(empty, device=grad.device)] == 0)), "empty experts must get zero gradients"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("add_bias", [False, True])
+@pytest.mark.parametrize("activation", ["swiglu", "gelu", "silu"])
+def test_empty_batch(activation, add_bias, dtype):
+    """No tokens at all: outputs of shape (0, H) and (0, E), an input gradient of shape (0, H), and weight and bias
+    gradients that are exact zeros (every expert is empty), on the fused pipelines and on the one that runs an
+    arbitrary callable between two plain grouped GEMMs."""
+
+    E, k, H, I = 4, 2, 64, 32
+    act = {"swiglu": xma.swiglu_packed, "gelu": nn.GELU(approximate="tanh"), "silu": nn.SiLU()}[activation]
+    moe = xma.MoE(E, k, H, I, act, activation == "swiglu", add_bias, 0.02).to(dtype).cuda()
+    x = torch.randn(0, H, device="cuda").to(dtype).requires_grad_()
+    y, logits = moe(x)
+    assert y.shape == (0, H) and logits.shape == (0, E)
+    y.sum().backward()  # an expanded gradient without rows
+    assert x.grad.shape == (0, H)
+    for name, p in moe.named_parameters():
+        assert p.grad is not None and p.grad.shape == p.shape and not bool(p.grad.any()), name
+
+
 def test_backward_of_an_expanded_gradient():
     """y.mean(0) upstream hands backward a gradient with strides (0, 1): it must be made dense, not rejected."""
 

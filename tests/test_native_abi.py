@@ -72,7 +72,7 @@ def test_identification_and_error_channel():
     assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "struct_size" in _native.last_error()
     args.struct_size = ctypes.sizeof(args)
     assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "num_experts" in _native.last_error()
-    args.num_experts, args.n, args.k, args.lda = 4, 12, 64, 32  # row stride of A shorter than the reduction
+    args.num_experts, args.n, args.k, args.lda, args.rows = 4, 12, 64, 32, 16  # row stride of A shorter than the reduction
     off = (ctypes.c_int32 * 5)()
     args.expert_offsets = ctypes.cast(off, ctypes.c_void_p)
     assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "lda too small" in _native.last_error()
