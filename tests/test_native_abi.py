@@ -206,3 +206,33 @@ def test_product_sources_never_touch_the_oracle():
                     if re.search(r"\boracle\b", text):
                         offenders.append(os.path.join(folder, name))
     assert offenders == []
+
+
+def test_header_is_plain_c_and_links(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 with no extension, and a C program linked against the
+    library reads the same interface version as the header it was compiled with (no GPU call)."""
+
+    import shutil
+    import subprocess
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib_dir = os.path.join(root, "flash_model_architectures_amd", "lib")
+    source = tmp_path / "abi.c"
+    source.write_text(
+        '#include "xma_hip.h"\n'
+        "int main(void) {\n"
+        "    xma_grouped_gemm_args a;\n"
+        "    a.struct_size = (uint32_t)sizeof a;\n"
+        "    return a.struct_size != 0 && xma_abi_version() == XMA_ABI_VERSION ? 0 : 1;\n"
+        "}\n"
+    )
+    exe = tmp_path / "abi"
+    subprocess.run(
+        ["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(root, "include"), str(source),
+         "-L", lib_dir, "-lxma_hip", f"-Wl,-rpath,{lib_dir}", "-Wl,-rpath,/opt/rocm/lib", "-o", str(exe)],
+        check=True,
+    )
+    assert subprocess.run([str(exe)]).returncode == 0
+
