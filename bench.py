@@ -243,6 +243,10 @@ def _other_config(workload: dict, steps: int, warmup: int) -> dict:
         logits = moe.gate(x)
         _, selected = xma.topk_softmax(logits, k)
         counts = xma.route_tokens(selected, E).expert_frequency.cpu().to(torch.int64)
+        # tokens whose k-th and (k+1)-th largest router logits are equal: the only place where the choice of
+        # experts rests on a tie rule (lower expert index here)
+        ranked = torch.sort(logits.float(), dim=-1, descending=True).values
+        ties = int((ranked[:, k - 1] == ranked[:, k]).sum()) if E > k else 0
     kernels = _kernel_table(timeline.summary(), steps)
     gemm_ms = sum(kr["ms_per_step"] for kr in kernels if kr["kernel"].startswith("xma_grouped_gemm"))
     flops = 18.0 * T * k * H * I
@@ -263,7 +267,9 @@ def _other_config(workload: dict, steps: int, warmup: int) -> dict:
                 "max": int(counts.max()),
                 "experts_under_256_rows": int((counts < 256).sum()),
                 "row_tiles_of_256": int(sum(math.ceil(c / 256) for c in counts.tolist())),
+                "per_expert": counts.tolist(),
             },
+            "tokens_with_a_tie_at_the_selection_boundary": ties,
             "kernels": kernels,
         }
     )
