@@ -377,11 +377,19 @@ struct Kernel {
 
     // One phase = one 32-deep block = MI * NI matrix instructions of 16 cycles.  A wave that is alone on its SIMD
     // has nobody to hide its stalls, so the three instruction streams are interleaved by hand: the phase is cut into
-    // 16 slots of four matrix instructions (one A block against half of the B blocks); every slot also reads its share
-    // of the NEXT block's fragments (in the order the next phase needs them: all B blocks within the first slots, then
-    // the A blocks) and every other slot issues one DMA load.  The matrix instructions are inline assembly, which the
-    // instruction scheduler cannot classify, so the order is pinned with a scheduling fence after each slot.
-    // RP / RKB: ring position and block of the fragments being read; LP / LPH: the step and phase whose loads go out.
+    // 32 slots of two matrix instructions (one B block against two A blocks).  Every odd slot also reads one block
+    // of the NEXT phase's fragments and every fourth slot issues one DMA load.  The matrix instructions are inline
+    // assembly, which the instruction scheduler cannot classify, so the order is pinned with a scheduling fence
+    // after each slot.  RP / RKB: ring position and block of the fragments being read; LP / LPH: the step and phase
+    // whose loads go out.
+    //
+    // The granularity and the placement are measured choices (benchmark layer, all launches of a pass, same
+    // session): against 16 slots of four instructions with the B blocks read two per slot in the first four slots
+    // and the loads in the odd slots, this schedule is 3.3 % faster; with the loads in slot 1 instead of slot 0 of
+    // every four 2.6 %; 16 slots with the reads spread out and the loads in even slots 1.4 %.  The kinds differ in
+    // the best order of the reads: all A blocks, then all B blocks where both operands cost the same number of LDS
+    // instructions (TN, MT), alternating where the transposed operand costs twice as many (NN).  One instruction
+    // per slot does not compile (the compiler runs out of scalar registers).
     //
     // The tail tile of an expert's rows runs exactly the same instruction stream on zeros for the rows that do not
     // exist.  Skipping the missing 16-row blocks was measured and is a LOSS: the 32 work-groups an XCD runs at a
@@ -391,21 +399,24 @@ struct Kernel {
     // (8 tail tiles among 67 at the benchmark shape).
     template <int RP, int LP, int LPH, bool MASKED>
     __device__ __forceinline__ void phase(int rkb, int cur, int64_t s, f32x4_t (&acc)[MI][NI]) {
-        constexpr int SLOTS = 2 * MI;  // 16
+        constexpr int SLOTS = 4 * MI;  // 32
         const int nxt = cur ^ 1;
 #pragma unroll
         for (int slot = 0; slot < SLOTS; ++slot) {
-            const int mi = slot / 2, n0 = (slot & 1) * (NI / 2);
-#pragma unroll
-            for (int j = 0; j < NI / 2; ++j) Mma16<T>::run(fb[cur][n0 + j], fa[cur][mi], acc[mi][n0 + j]);
-            // next block's fragments: slots 0-3 read two B blocks each, slots 4-11 one A block each
-            if (slot < 4) {
-                fb[nxt][2 * slot] = read_b<RP>(rkb, 2 * slot);
-                fb[nxt][2 * slot + 1] = read_b<RP>(rkb, 2 * slot + 1);
-            } else if (slot < 4 + MI) {
-                fa[nxt][slot - 4] = read_a<RP>(rkb, slot - 4);
+            const int ni = slot / 4, m0 = (slot & 3) * 2;
+            Mma16<T>::run(fb[cur][ni], fa[cur][m0], acc[m0][ni]);
+            Mma16<T>::run(fb[cur][ni], fa[cur][m0 + 1], acc[m0 + 1][ni]);
+            if (slot % 2 == 1) {
+                const int r = slot / 2;  // the r-th of the 16 fragment blocks of the next phase
+                if constexpr (KIND == XMA_GEMM_NN) {
+                    if (r % 2 == 0) fa[nxt][r / 2] = read_a<RP>(rkb, r / 2);
+                    else fb[nxt][r / 2] = read_b<RP>(rkb, r / 2);
+                } else {
+                    if (r < MI) fa[nxt][r] = read_a<RP>(rkb, r);
+                    else fb[nxt][r - MI] = read_b<RP>(rkb, r - MI);
+                }
             }
-            if (slot % 2 == 1) issue_slot<LP, LPH, MASKED>(slot / 2, s);
+            if (slot % 4 == 0) issue_slot<LP, LPH, MASKED>(slot / 4, s);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
