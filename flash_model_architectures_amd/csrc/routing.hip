@@ -3,19 +3,20 @@
 // backward).  All integer results are order-independent or explicitly ordered, so they are
 // bit-exact from run to run.
 //
-// Work decomposition of the counting sort: the id stream is cut into contiguous chunks of
-// kChunk ids, one wavefront per chunk.  (1) every wave builds a private histogram of its
-// chunk in LDS and writes it out as a row of `unit_hist[units][E]`; (2) a column-wise
-// exclusive scan over the units plus an exclusive scan over the experts turn the rows into
-// the first output slot of every (unit, expert) pair; (3) every wave walks its chunk again in
-// order, ranks equal ids inside each 64-wide batch with ballots, and writes the permutation.
+// Work decomposition of the counting sort: the id stream is cut into contiguous chunks ("units") of
+// kChunk ids.  (1) the histogram of every unit is built in LDS and written out as a row of
+// `unit_hist[units][E]`; (2) a column-wise exclusive scan over the units plus an exclusive scan
+// over the experts turn the rows into the first output slot of every (unit, expert) pair; (3) the
+// unit is walked again in order, equal ids inside each 64-wide batch are ranked with ballots, and
+// the permutation is written.  For the sizes of an MoE layer a unit belongs to a block of four
+// waves (a quarter each) and steps (2) and (3) are one kernel; beyond, a unit belongs to one wave.
 #include <mutex>
 
 #include "common.h"
 
 namespace xma {
 
-constexpr int kChunk = 1024;        // ids per wave-unit of the counting sort
+constexpr int kChunk = 1024;        // ids per unit of the counting sort
 constexpr int kMaxExperts = 16384;  // same limit as the reference kernel (forward.cu:12)
 
 // Working memory of xma_route_build_static, the entry point that allocates nothing: the per-chunk histograms
@@ -121,11 +122,11 @@ __global__ __launch_bounds__(1024) void count_single_block_kernel(const IdT* __r
 // A wave reads its ids kChunk at a time: 16 per lane, requested together (the walk over a chunk is otherwise a chain
 // of dependent load latencies), -1 past `end`.
 constexpr int kBatches = kChunk / kWaveSize;
-template <typename IdT>
+template <typename IdT, int BATCHES>
 __device__ __forceinline__ void load_chunk(const IdT* __restrict__ ids, int64_t begin, int64_t end, int lane,
-                                           int64_t (&v)[kBatches]) {
+                                           int64_t (&v)[BATCHES]) {
 #pragma unroll
-    for (int j = 0; j < kBatches; ++j) {
+    for (int j = 0; j < BATCHES; ++j) {
         const int64_t i = begin + j * kWaveSize + lane;
         v[j] = i < end ? (int64_t)ids[i] : -1;
     }
@@ -180,6 +181,34 @@ __global__ __launch_bounds__(256) void unit_hist_kernel(const IdT* __restrict__ 
         uint32_t* row = unit_hist + unit * E;
         for (int i = lane; i < E; i += kWaveSize) row[i] = mine[i];
     }
+}
+
+// The same table of per-unit histograms, written by one block of four waves per unit: a wave counts a quarter of the
+// unit (four batches instead of sixteen in a row), the block adds the four rows up.  First launch of the two-launch
+// counting sort.
+constexpr int kQuarter = kChunk / 4;                  // ids per wave when four waves share a unit
+constexpr int kQuarterBatches = kQuarter / kWaveSize;  // 4
+template <typename IdT>
+__global__ __launch_bounds__(256) void block_hist_kernel(const IdT* __restrict__ ids, int64_t n, int E,
+                                                          uint32_t* __restrict__ unit_hist) {
+    extern __shared__ uint32_t lds_hist[];  // [4][E]
+    const int wave = threadIdx.x / kWaveSize;
+    const int lane = lane_id();
+    const int64_t unit = blockIdx.x;
+    const int64_t begin = unit * kChunk + wave * kQuarter;
+    const int64_t end = begin + kQuarter < n ? begin + kQuarter : n;
+    int64_t v[kQuarterBatches];
+    load_chunk(ids, begin < n ? begin : n, end, lane, v);  // requested before the LDS rows are cleared (all -1 past n)
+    for (int i = threadIdx.x; i < 4 * E; i += 256) lds_hist[i] = 0;
+    __syncthreads();
+    uint32_t* mine = lds_hist + wave * E;
+#pragma unroll
+    for (int j = 0; j < kQuarterBatches; ++j)
+        if (v[j] >= 0 && v[j] < E) atomicAdd(&mine[v[j]], 1u);
+    __syncthreads();
+    uint32_t* row = unit_hist + unit * E;
+    for (int i = threadIdx.x; i < E; i += 256)
+        row[i] = lds_hist[i] + lds_hist[E + i] + lds_hist[2 * E + i] + lds_hist[3 * E + i];
 }
 
 // One block of 16 waves per 64 experts: lane = expert column, wave = a segment of the units.
@@ -304,15 +333,55 @@ __global__ __launch_bounds__(256) void place_kernel(const IdT* __restrict__ ids,
         place_batch(v[j], begin + j * kWaveSize + lane, E, nbits, lane, next, sorted_ids, perm);
 }
 
+// Column sums of the table of per-unit histograms, by one block of 256 threads: total[e] += all units, before[e] +=
+// the units before `unit`.  A thread handles V adjacent experts (one 4 * V-byte load per unit) of the units r,
+// r + rows, ...; the number of thread columns is E / V rounded up to a power of two, so consecutive lanes read
+// consecutive words.  Every load of a thread is requested before the first is used when the table has at most
+// kInFlight * rows units.
+template <int V>
+__device__ __forceinline__ void sum_table(const uint32_t* __restrict__ unit_hist, int64_t units, int64_t unit, int E,
+                                          uint32_t* total, uint32_t* before) {
+    typedef uint32_t vec_t __attribute__((ext_vector_type(V)));
+    constexpr int kInFlight = V == 4 ? 16 : 32;
+    const int groups = E / V;
+    int cols = 1;
+    while (cols < groups) cols <<= 1;
+    const int rows = 256 / cols;  // E <= 256
+    const int c = threadIdx.x & (cols - 1);
+    const int r = threadIdx.x / cols;
+    if (c >= groups) return;
+    const vec_t* table = reinterpret_cast<const vec_t*>(unit_hist) + c;
+    vec_t all = 0, mine = 0;
+    for (int64_t u0 = r; u0 < units; u0 += (int64_t)rows * kInFlight) {
+        vec_t h[kInFlight];
+#pragma unroll
+        for (int j = 0; j < kInFlight; ++j) {
+            const int64_t u = u0 + (int64_t)j * rows;
+            h[j] = u < units ? table[u * groups] : vec_t(0);
+        }
+#pragma unroll
+        for (int j = 0; j < kInFlight; ++j) {
+            const int64_t u = u0 + (int64_t)j * rows;
+            all += h[j];
+            mine += u < unit ? h[j] : vec_t(0);
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < V; ++q) {
+        atomicAdd(&total[c * V + q], (uint32_t)all[q]);
+        atomicAdd(&before[c * V + q], (uint32_t)mine[q]);
+    }
+}
+
 // Second and last launch of the counting sort for the sizes of an MoE layer (units * E <= kFusedScanValues, E <= 256;
-// the first launch is unit_hist_kernel).  One work-group moves data at a small fraction of the device's rate, so
-// the ids are spread over many small blocks, four waves = four units each, and every block repeats the scan for
+// the first launch is block_hist_kernel).  One work-group moves data at a small fraction of the device's rate, so
+// the ids are spread over many small blocks, one unit of four waves each, and every block repeats the scan for
 // itself: it reads the whole table of per-unit histograms (at most 64 KiB, L2-resident) and adds up, per expert,
 // all units (the expert's total) and the units before its own (where its ids start inside the expert's range);
-// thread e scans the totals into the offsets with wave shuffles; then every wave places the ids of its unit, which
-// it requested before the scan began.  Block 0 also writes counts and offsets.
+// thread e scans the totals into the offsets with wave shuffles; then every wave places its quarter of the unit,
+// which it requested before the scan began and counted for itself while the table was on its way (a wave's ids
+// start after those of the waves before it).  Block 0 also writes counts and offsets.
 constexpr int kFusedScanValues = 16384;
-constexpr int kFusedUnitsPerBlock = 4;
 template <typename IdT, typename OutT>
 __global__ __launch_bounds__(256) void scan_place_kernel(const IdT* __restrict__ ids, int64_t n, int E, int nbits,
                                                           int64_t units, const uint32_t* __restrict__ unit_hist,
@@ -322,54 +391,30 @@ __global__ __launch_bounds__(256) void scan_place_kernel(const IdT* __restrict__
     uint32_t* total = lds_hist;
     uint32_t* before = lds_hist + E;
     uint32_t* next_all = lds_hist + 2 * E;
-    uint32_t* wave_sum = lds_hist + (2 + kFusedUnitsPerBlock) * E;
+    uint32_t* wave_sum = lds_hist + 6 * E;
     const int wave = threadIdx.x / kWaveSize;
     const int lane = lane_id();
-    const int64_t first_unit = (int64_t)blockIdx.x * kFusedUnitsPerBlock;
+    const int64_t unit = blockIdx.x;
 
-    // this wave's ids, on their way while the scan runs
-    const int64_t begin = (first_unit + wave) * kChunk;
-    const int64_t end = begin + kChunk < n ? begin + kChunk : n;
-    int64_t v[kBatches];
-    load_chunk(ids, begin, end, lane, v);  // all -1 for a unit past the end
-    // ... and so are the histograms of the block's own units (thread e: expert e), which are needed after the scan
-    uint32_t own[kFusedUnitsPerBlock];
-#pragma unroll
-    for (int w = 0; w < kFusedUnitsPerBlock; ++w)
-        own[w] = (int)threadIdx.x < E && first_unit + w < units ? unit_hist[(first_unit + w) * E + threadIdx.x] : 0u;
+    // this wave's ids, on their way while the table is read
+    const int64_t begin = unit * kChunk + wave * kQuarter;
+    const int64_t end = begin + kQuarter < n ? begin + kQuarter : n;
+    int64_t v[kQuarterBatches];
+    load_chunk(ids, begin < n ? begin : n, end, lane, v);  // all -1 for a quarter past the end
 
-    for (int i = threadIdx.x; i < 2 * E; i += 256) lds_hist[i] = 0;
+    for (int i = threadIdx.x; i < 6 * E; i += 256) lds_hist[i] = 0;
     __syncthreads();
 
-    // Thread (r, c) adds up column c (+ cols, + 2 cols ...) of the table over the units r, r + rows, ...; cols is E
-    // rounded up to a power of two, so consecutive lanes read consecutive words.
+    // the wave's own histogram (its quarter of the unit) ...
     {
-        int cols = 1;
-        while (cols < E) cols <<= 1;
-        const int rows = 256 / cols;  // E <= 256
-        const int c = threadIdx.x & (cols - 1);
-        const int r = threadIdx.x / cols;
-        if (c < E) {
-            constexpr int kInFlight = 16;
-            uint32_t all = 0, mine = 0;
-            for (int64_t u0 = r; u0 < units; u0 += (int64_t)rows * kInFlight) {
-                uint32_t h[kInFlight];
+        uint32_t* own = next_all + wave * E;
 #pragma unroll
-                for (int j = 0; j < kInFlight; ++j) {
-                    const int64_t u = u0 + (int64_t)j * rows;
-                    h[j] = u < units ? unit_hist[u * E + c] : 0u;
-                }
-#pragma unroll
-                for (int j = 0; j < kInFlight; ++j) {
-                    const int64_t u = u0 + (int64_t)j * rows;
-                    all += h[j];
-                    mine += u < first_unit ? h[j] : 0u;
-                }
-            }
-            atomicAdd(&total[c], all);
-            atomicAdd(&before[c], mine);
-        }
+        for (int j = 0; j < kQuarterBatches; ++j)
+            if (v[j] >= 0 && v[j] < E) atomicAdd(&own[v[j]], 1u);
     }
+    // ... and the column sums of the table: 16-byte loads when a row is a whole number of them
+    if (E % 4 == 0 && (reinterpret_cast<uintptr_t>(unit_hist) & 15) == 0) sum_table<4>(unit_hist, units, unit, E, total, before);
+    else sum_table<1>(unit_hist, units, unit, E, total, before);
     __syncthreads();
 
     // exclusive scan of the totals over the experts: thread e holds expert e
@@ -391,12 +436,13 @@ __global__ __launch_bounds__(256) void scan_place_kernel(const IdT* __restrict__
             offsets[e] = (int32_t)first_slot;
             if (e == E - 1) offsets[E] = (int32_t)(first_slot + count);
         }
-        // first output slot of the ids of expert e in each of the block's units
+        // first output slot of the ids of expert e in each of the block's waves
         uint32_t slot = first_slot + before[e];
 #pragma unroll
-        for (int w = 0; w < kFusedUnitsPerBlock; ++w) {
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t own_count = next_all[w * E + e];
             next_all[w * E + e] = slot;
-            slot += own[w];
+            slot += own_count;
         }
     }
     __syncthreads();
@@ -404,7 +450,7 @@ __global__ __launch_bounds__(256) void scan_place_kernel(const IdT* __restrict__
     if (begin >= n) return;
     uint32_t* next = next_all + wave * E;
 #pragma unroll
-    for (int j = 0; j < kBatches; ++j)
+    for (int j = 0; j < kQuarterBatches; ++j)
         place_batch(v[j], begin + j * kWaveSize + lane, E, nbits, lane, next, sorted_ids, perm);
 }
 
@@ -749,21 +795,18 @@ static int route_build_launch(const void* ids, int ids_is_i64, int64_t n, int32_
         return check_launch("xma_route_build");
     }
     const int64_t units = ceil_div(n, kChunk);
-    const int wpb = sort_waves_per_block(E);
-    const unsigned blocks = (unsigned)ceil_div(units, wpb);
-    const size_t lds = (size_t)wpb * E * sizeof(uint32_t);
     uint32_t* unit_hist = (uint32_t*)workspace;
-    if (ids_is_i64)
-        hipLaunchKernelGGL(unit_hist_kernel<int64_t>, dim3(blocks), dim3(wpb * kWaveSize), lds, stream,
-                           (const int64_t*)ids, n, (int)E, wpb, unit_hist);
-    else
-        hipLaunchKernelGGL(unit_hist_kernel<int32_t>, dim3(blocks), dim3(wpb * kWaveSize), lds, stream,
-                           (const int32_t*)ids, n, (int)E, wpb, unit_hist);
-    if (units * E <= kFusedScanValues && E <= 256) {  // second and last launch: scan and placement in one
-        const unsigned place_blocks = (unsigned)ceil_div(units, kFusedUnitsPerBlock);
-        const size_t place_lds = ((size_t)(2 + kFusedUnitsPerBlock) * E + kFusedUnitsPerBlock) * sizeof(uint32_t);
+    if (units * E <= kFusedScanValues && E <= 256) {  // two launches: histograms, then scan and placement in one
+        const size_t hist_lds = (size_t)4 * E * sizeof(uint32_t);
+        if (ids_is_i64)
+            hipLaunchKernelGGL(block_hist_kernel<int64_t>, dim3((unsigned)units), dim3(256), hist_lds, stream,
+                               (const int64_t*)ids, n, (int)E, unit_hist);
+        else
+            hipLaunchKernelGGL(block_hist_kernel<int32_t>, dim3((unsigned)units), dim3(256), hist_lds, stream,
+                               (const int32_t*)ids, n, (int)E, unit_hist);
+        const size_t place_lds = ((size_t)6 * E + 4) * sizeof(uint32_t);
 #define XMA_SCAN_PLACE(IdT, OutT)                                                                                   \
-    hipLaunchKernelGGL((scan_place_kernel<IdT, OutT>), dim3(place_blocks), dim3(256), place_lds, stream,             \
+    hipLaunchKernelGGL((scan_place_kernel<IdT, OutT>), dim3((unsigned)units), dim3(256), place_lds, stream,          \
                        (const IdT*)ids, n, (int)E, nbits, units, (const uint32_t*)unit_hist, counts, offsets,       \
                        (OutT*)sorted_ids, (OutT*)perm)
         if (ids_is_i64) {
@@ -780,6 +823,15 @@ static int route_build_launch(const void* ids, int ids_is_i64, int64_t n, int32_
 #undef XMA_SCAN_PLACE
         return check_launch("xma_route_build");
     }
+    const int wpb = sort_waves_per_block(E);
+    const unsigned blocks = (unsigned)ceil_div(units, wpb);
+    const size_t lds = (size_t)wpb * E * sizeof(uint32_t);
+    if (ids_is_i64)
+        hipLaunchKernelGGL(unit_hist_kernel<int64_t>, dim3(blocks), dim3(wpb * kWaveSize), lds, stream,
+                           (const int64_t*)ids, n, (int)E, wpb, unit_hist);
+    else
+        hipLaunchKernelGGL(unit_hist_kernel<int32_t>, dim3(blocks), dim3(wpb * kWaveSize), lds, stream,
+                           (const int32_t*)ids, n, (int)E, wpb, unit_hist);
     hipLaunchKernelGGL(unit_scan_kernel, dim3((E + kWaveSize - 1) / kWaveSize), dim3(1024), 0, stream, unit_hist, units,
                        (int)E, counts);
     hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, stream, (const uint32_t*)counts, (int)E, offsets);
