@@ -549,32 +549,49 @@ __device__ __forceinline__ float key_to_float(uint32_t key) {
     return __uint_as_float((key & 0x80000000u) ? (key ^ 0x80000000u) : ~key);
 }
 
+// Maximum / sum over the aligned group of `width` lanes (a power of two) that the lane belongs to.
+__device__ __forceinline__ uint64_t max_with_lane_xor(uint64_t v, int off) {
+    uint32_t lo = __shfl_xor((uint32_t)v, off, kWaveSize);
+    uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, kWaveSize);
+    uint64_t o = ((uint64_t)hi << 32) | lo;
+    return o > v ? o : v;
+}
 __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
 #pragma unroll
-    for (int off = kWaveSize / 2; off > 0; off >>= 1) {
-        uint32_t lo = __shfl_xor((uint32_t)v, off, kWaveSize);
-        uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, kWaveSize);
-        uint64_t o = ((uint64_t)hi << 32) | lo;
-        v = o > v ? o : v;
-    }
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) v = max_with_lane_xor(v, off);
+    return v;
+}
+__device__ __forceinline__ uint64_t group_max_u64(uint64_t v, int width) {
+    if (width == kWaveSize) return wave_max_u64(v);  // constant lane offsets
+    for (int off = width / 2; off > 0; off >>= 1) v = max_with_lane_xor(v, off);
+    return v;
+}
+__device__ __forceinline__ float group_sum(float v, int width) {
+    for (int off = width / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWaveSize);
     return v;
 }
 
-// One wave per token; lane l owns experts l, l+64, ...  (EPL per lane, E <= 64*EPL).
+// A group of G lanes per token (G a power of two, k <= G, E <= G * EPL), 64 / G tokens per wave; lane g of the group
+// owns experts g, g + G, ...  A round costs EPL compare-and-selects per lane and log2(G) exchange steps, so few lanes
+// with many experts each are cheaper than a whole wave per token (E = 64: 8 lanes x 8 experts).
 // key = (order_key(value) << 32) | (0xffffffff - expert): the maximum picks the largest value
 // and, among equals, the lowest expert index.
 template <typename T, int EPL, typename IdxT>
-__global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__ logits, int64_t Tn, int E, int k,
+__global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__ logits, int64_t Tn, int E, int k, int G,
                                                             int64_t ld, T* __restrict__ weights,
                                                             IdxT* __restrict__ idx) {
     const int lane = lane_id();
-    const int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize;
-    if (t >= Tn) return;
-    const T* row = logits + t * ld;
+    const int g = lane & (G - 1);
+    const int tokens_per_wave = kWaveSize / G;
+    const int64_t first = ((int64_t)blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize) * tokens_per_wave;
+    if (first >= Tn) return;  // whole waves only: every lane of a wave takes part in the exchanges
+    const int64_t t = first + lane / G;
+    const bool live = t < Tn;
+    const T* row = logits + (live ? t : first) * ld;
     uint64_t keys[EPL];
 #pragma unroll
     for (int j = 0; j < EPL; ++j) {
-        const int e = lane + j * kWaveSize;
+        const int e = g + j * G;
         keys[j] = e < E ? (((uint64_t)order_key(Elem<T>::load(row + e)) << 32) | (uint32_t)(0xffffffffu - (uint32_t)e))
                         : 0ull;
     }
@@ -585,22 +602,22 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__
         uint64_t best = 0;
 #pragma unroll
         for (int j = 0; j < EPL; ++j) best = keys[j] > best ? keys[j] : best;
-        best = wave_max_u64(best);
+        best = group_max_u64(best, G);
 #pragma unroll
         for (int j = 0; j < EPL; ++j)
             if (keys[j] == best) keys[j] = 0ull;
         const float v = key_to_float((uint32_t)(best >> 32));
         if (s == 0) vmax = v;
-        if (lane == s) {
+        if (g == s) {
             my_val = v;
             my_idx = 0xffffffffu - (uint32_t)best;
         }
     }
-    const float ex = lane < k ? expf(my_val - vmax) : 0.0f;
-    const float denom = wave_sum(ex);
-    if (lane < k) {
-        Elem<T>::store(weights + t * k + lane, ex / denom);
-        idx[t * k + lane] = (IdxT)my_idx;
+    const float ex = g < k ? expf(my_val - vmax) : 0.0f;
+    const float denom = group_sum(ex, G);
+    if (live && g < k) {
+        Elem<T>::store(weights + t * k + g, ex / denom);
+        idx[t * k + g] = (IdxT)my_idx;
     }
 }
 
@@ -646,34 +663,37 @@ __global__ __launch_bounds__(64) void topk_softmax_lds_kernel(const T* __restric
 }
 
 // d_logits[t, :] = 0, then d_logits[t, idx[t, j]] = w_j * (dw_j - sum_i w_i dw_i) with
-// w = softmax(logits[t, idx[t, :]]) recomputed in fp32.  One wave per token.
+// w = softmax(logits[t, idx[t, :]]) recomputed in fp32.  A group of G lanes per token (a power of two, k <= G).
 template <typename T, typename IdxT>
 __global__ __launch_bounds__(256) void topk_softmax_bwd_kernel(const T* __restrict__ logits, int64_t ld_logits,
                                                                 const T* __restrict__ d_weights,
                                                                 const IdxT* __restrict__ idx, int64_t Tn, int E, int k,
-                                                                T* __restrict__ d_logits, int64_t ld) {
+                                                                int G, T* __restrict__ d_logits, int64_t ld) {
     const int lane = lane_id();
-    const int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize;
-    if (t >= Tn) return;
-    T* out = d_logits + t * ld;
-    for (int e = lane; e < E; e += kWaveSize) Elem<T>::store(out + e, 0.0f);
+    const int g = lane & (G - 1);
+    const int64_t first = ((int64_t)blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize) * (kWaveSize / G);
+    if (first >= Tn) return;  // whole waves only: every lane of a wave takes part in the exchanges
+    const int64_t t = first + lane / G;
+    const bool live = t < Tn;
+    T* out = d_logits + (live ? t : first) * ld;
+    if (live)
+        for (int e = g; e < E; e += G) Elem<T>::store(out + e, 0.0f);
     int64_t e_sel = 0;
     float v = -INFINITY, dw = 0.0f;
-    if (lane < k) {
-        e_sel = (int64_t)idx[t * k + lane];
+    if (live && g < k) {
+        e_sel = (int64_t)idx[t * k + g];
         v = Elem<T>::load(logits + t * ld_logits + e_sel);
-        dw = Elem<T>::load(d_weights + t * k + lane);
+        dw = Elem<T>::load(d_weights + t * k + g);
     }
     float vmax = v;
-#pragma unroll
-    for (int off = kWaveSize / 2; off > 0; off >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, off, kWaveSize));
-    const float ex = lane < k ? expf(v - vmax) : 0.0f;
-    const float w = ex / wave_sum(ex);
-    const float dot = wave_sum(w * dw);
+    for (int off = G / 2; off > 0; off >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, off, kWaveSize));
+    const float ex = live && g < k ? expf(v - vmax) : 0.0f;
+    const float w = ex / group_sum(ex, G);
+    const float dot = group_sum(w * dw, G);
     // the zero fill above and this store touch the same addresses from different lanes
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    if (lane < k) Elem<T>::store(out + e_sel, w * (dw - dot));
+    if (live && g < k) Elem<T>::store(out + e_sel, w * (dw - dot));
 }
 
 static int ceil_log2(int v) {
@@ -911,24 +931,29 @@ int xma_topk_softmax(const void* logits, int dtype, int64_t T, int32_t E, int32_
     XMA_REQUIRE(T >= 0 && ld >= E, "xma_topk_softmax: bad T=%lld or row stride %lld", (long long)T, (long long)ld);
     if (T == 0) return 0;
     XMA_REQUIRE(logits && weights && idx, "xma_topk_softmax: null pointer");
+    // lanes per token: at least k (lane s of a group keeps the s-th selection) and enough for eight experts per lane
+    int G = 1;
+    while (G < k) G <<= 1;
+    while (G < kWaveSize && G * 8 < E) G <<= 1;
+    const int per_lane = (int)ceil_div(E, G);
     const int wpb = 4;
-    const unsigned blocks = (unsigned)ceil_div(T, wpb);
+    const unsigned blocks = (unsigned)ceil_div(T, (int64_t)wpb * (kWaveSize / G));
 #define XMA_TOPK(T_, EPL, IdxT)                                                                                    \
     hipLaunchKernelGGL((topk_softmax_kernel<T_, EPL, IdxT>), dim3(blocks), dim3(wpb * kWaveSize), 0, stream,        \
-                       (const T_*)logits, T, (int)E, (int)k, ld, (T_*)weights, (IdxT*)idx)
+                       (const T_*)logits, T, (int)E, (int)k, G, ld, (T_*)weights, (IdxT*)idx)
 #define XMA_TOPK_E(T_, IdxT)                                                                                       \
-    if (E <= 64)                                                                                                   \
-        XMA_TOPK(T_, 1, IdxT);                                                                                     \
-    else if (E <= 128)                                                                                             \
-        XMA_TOPK(T_, 2, IdxT);                                                                                     \
-    else if (E <= 256)                                                                                             \
-        XMA_TOPK(T_, 4, IdxT);                                                                                     \
-    else if (E <= 512)                                                                                             \
-        XMA_TOPK(T_, 8, IdxT);                                                                                     \
-    else                                                                                                           \
+    if (E > 512)                                                                                                   \
         hipLaunchKernelGGL((topk_softmax_lds_kernel<T_, IdxT>), dim3((unsigned)T), dim3(kWaveSize),                \
                            (size_t)E * sizeof(uint32_t), stream, (const T_*)logits, T, (int)E, (int)k, ld,         \
-                           (T_*)weights, (IdxT*)idx)
+                           (T_*)weights, (IdxT*)idx);                                                              \
+    else if (per_lane <= 1)                                                                                        \
+        XMA_TOPK(T_, 1, IdxT);                                                                                     \
+    else if (per_lane <= 2)                                                                                        \
+        XMA_TOPK(T_, 2, IdxT);                                                                                     \
+    else if (per_lane <= 4)                                                                                        \
+        XMA_TOPK(T_, 4, IdxT);                                                                                     \
+    else                                                                                                           \
+        XMA_TOPK(T_, 8, IdxT)
     XMA_DISPATCH_DTYPE(dtype, T_, if (idx_is_i64) { XMA_TOPK_E(T_, int64_t); } else { XMA_TOPK_E(T_, int32_t); })
 #undef XMA_TOPK_E
 #undef XMA_TOPK
@@ -944,16 +969,19 @@ int xma_topk_softmax_bwd(const void* logits, int64_t ld_logits, const void* d_we
     XMA_REQUIRE(T >= 0 && ld >= E && ld_logits >= E, "xma_topk_softmax_bwd: bad T or row stride");
     if (T == 0) return 0;
     XMA_REQUIRE(logits && d_weights && idx && d_logits, "xma_topk_softmax_bwd: null pointer");
+    int G = 1;  // lanes per token: at least k, and at most eight zero stores per lane
+    while (G < k) G <<= 1;
+    while (G < kWaveSize && G * 8 < E) G <<= 1;
     const int wpb = 4;
-    const unsigned blocks = (unsigned)ceil_div(T, wpb);
+    const unsigned blocks = (unsigned)ceil_div(T, (int64_t)wpb * (kWaveSize / G));
     XMA_DISPATCH_DTYPE(
         dtype, T_,
         if (idx_is_i64) hipLaunchKernelGGL((topk_softmax_bwd_kernel<T_, int64_t>), dim3(blocks), dim3(wpb * kWaveSize),
                                            0, stream, (const T_*)logits, ld_logits, (const T_*)d_weights,
-                                           (const int64_t*)idx, T, (int)E, (int)k, (T_*)d_logits, ld);
+                                           (const int64_t*)idx, T, (int)E, (int)k, G, (T_*)d_logits, ld);
         else hipLaunchKernelGGL((topk_softmax_bwd_kernel<T_, int32_t>), dim3(blocks), dim3(wpb * kWaveSize), 0, stream,
                                 (const T_*)logits, ld_logits, (const T_*)d_weights, (const int32_t*)idx, T, (int)E,
-                                (int)k, (T_*)d_logits, ld))
+                                (int)k, G, (T_*)d_logits, ld))
     return check_launch("xma_topk_softmax_bwd");
 }
 
