@@ -106,6 +106,11 @@ PROTOTYPES: dict[str, tuple] = {
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int32, c_int64, c_int, c_void_p],
     ),
+    "xma_router_weight_grad_workspace_bytes": (c_int64, [c_int64, c_int32, c_int64]),
+    "xma_router_weight_grad": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int64, c_int32, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p],
+    ),
     "xma_pack_sequence": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p],

@@ -21,7 +21,7 @@ CSRC_DIR = os.path.join(_PACKAGE_DIR, "csrc")
 LIB_DIR = os.path.join(_PACKAGE_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libxma_hip.so")
 
-SOURCES = ["common.hip", "routing.hip", "rowmove.hip", "seqpack.hip", "bias.hip", "swiglu.hip", "grouped_gemm.hip", "grouped_gemm_dma.hip"]
+SOURCES = ["common.hip", "routing.hip", "rowmove.hip", "seqpack.hip", "bias.hip", "swiglu.hip", "router_wgrad.hip", "grouped_gemm.hip", "grouped_gemm_dma.hip"]
 
 # packed-fp32 VALU forms are switched off for every kernel in this library
 HIPCC_FLAGS = [

@@ -31,10 +31,44 @@ from ..ops import (
     gate_grad,
     group,
     group_bwd_W,
+    router_weight_grad,
     scatter2scatter,
     up_projection_fused,
 )
 from ..utils import XMAModule
+
+
+class _GateLinear(torch.autograd.Function):
+    """router_logits = x @ weight^T (xma/layers/moe/__init__.py:148,192).  Forward and input gradient are the library's
+    GEMMs; the weight gradient, a [num_experts, hidden] output reduced over every token, goes through
+    `router_weight_grad` (a hand-written kernel for 16-bit types and num_experts a multiple of 8 up to 256, the library
+    otherwise)."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        ctx.save_for_backward(x, weight)
+        return torch.nn.functional.linear(x, weight)
+
+    @staticmethod
+    def backward(ctx, d_logits: torch.Tensor):
+        x, weight = ctx.saved_tensors
+        d_x = d_weight = None
+        if ctx.needs_input_grad[0]:
+            d_x = d_logits @ weight
+        if ctx.needs_input_grad[1]:
+            d_weight = torch.empty_like(weight, memory_format=torch.contiguous_format)
+            router_weight_grad(x=x, d_logits=d_logits.contiguous(), d_weight=d_weight)
+        return d_x, d_weight
+
+
+class _Gate(nn.Linear):
+    """The router's linear layer (nn.Linear in the reference, xma/layers/moe/__init__.py:148): same parameters and
+    state_dict, forward through `_GateLinear` (module hooks still apply)."""
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        if self.bias is not None or input.dim() != 2:
+            return super().forward(input)
+        return _GateLinear.apply(input, self.weight)
 
 
 class _ScatteredExperts(torch.autograd.Function):
@@ -444,7 +478,7 @@ class MoE(XMAModule):
         self.intermediate_size = intermediate_size
         self.is_glu = is_glu
 
-        self.gate = nn.Linear(in_features=hidden_size, out_features=num_experts, bias=False)
+        self.gate = _Gate(in_features=hidden_size, out_features=num_experts, bias=False)
         self.c_fc = Experts(
             num_experts=num_experts,
             in_features=hidden_size,

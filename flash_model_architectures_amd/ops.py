@@ -336,6 +336,59 @@ def gate_grad(expanded: torch.Tensor, grad_out: torch.Tensor, d_gates: torch.Ten
     )
 
 
+def router_weight_grad_supported(x: torch.Tensor, d_logits: torch.Tensor) -> bool:
+    """True when the hand-written kernel behind `router_weight_grad` takes these operands (16-bit element types, E a
+    multiple of 8 up to 256, H a multiple of 8, 16-byte aligned rows); other shapes go to the library's GEMM."""
+
+    if x.dtype not in (torch.bfloat16, torch.float16) or d_logits.dtype != x.dtype or x.dim() != 2 or d_logits.dim() != 2:
+        return False
+    E, H = d_logits.size(1), x.size(1)
+    if E % 8 != 0 or E > 256 or H % 8 != 0 or x.size(0) != d_logits.size(0):
+        return False
+    for t in (x, d_logits):
+        if t.size(0) > 0 and (t.stride(1) != 1 or t.stride(0) % 8 != 0 or t.data_ptr() % 16 != 0):
+            return False
+    return True
+
+
+@xma_op(mutates_args={"d_weight"})
+def router_weight_grad(x: torch.Tensor, d_logits: torch.Tensor, d_weight: torch.Tensor) -> None:
+    """d_weight[E, H] = d_logits[T, E]^T x[T, H] with fp32 accumulation: the weight gradient of the gate's linear layer
+    (xma/layers/moe/__init__.py:148,192).  Shapes the kernel does not take (`router_weight_grad_supported`) are one
+    library GEMM, as in the reference."""
+
+    nat.require_device(x, d_logits, d_weight)
+    T, H = x.shape
+    E = d_logits.size(1)
+    assert d_logits.size(0) == T and d_weight.shape == (E, H) and d_weight.stride(1) == 1
+    assert d_weight.dtype == x.dtype == d_logits.dtype
+    if not router_weight_grad_supported(x, d_logits):
+        if d_weight.is_contiguous():
+            torch.matmul(d_logits.t(), x, out=d_weight)
+        else:
+            d_weight.copy_(d_logits.t() @ x)
+        return
+    ws_bytes = nat.load().xma_router_weight_grad_workspace_bytes(T, E, H)
+    workspace = _workspace(x.device, ws_bytes)
+    nat.call(
+        "xma_router_weight_grad",
+        x.data_ptr(),
+        _row_stride(x),
+        d_logits.data_ptr(),
+        _row_stride(d_logits),
+        nat.dtype_code(x),
+        T,
+        E,
+        H,
+        d_weight.data_ptr(),
+        _row_stride(d_weight),
+        workspace.data_ptr(),
+        workspace.numel(),
+        nat.stream(),
+        nbytes=(x.numel() + d_logits.numel() + d_weight.numel()) * x.element_size(),
+    )
+
+
 @xma_op(mutates_args={"y"})
 def add_expert_bias(
     y: torch.Tensor, bias: torch.Tensor, sorted_expert_idxs: torch.Tensor, out_index: torch.Tensor | None = None

@@ -227,6 +227,19 @@ int xma_gate_grad(const void* y_exp, int64_t ld_exp, const void* dy, int64_t ld_
                   int64_t T, int32_t k, int64_t cols, int dtype, void* stream);
 
 /*
+ * Weight gradient of the router's linear layer: dw[E, H] = d_logits[T, E]^T x[T, H], fp32 accumulation in a
+ * fixed order (the token range is split over many blocks; the partial sums are added in split order).
+ * XMA_BF16 / XMA_F16 only; E a multiple of 8, at most 256; H a multiple of 8; ldx, ldd multiples of 8 and
+ * x, d_logits 16-byte aligned; ldw >= H.  T = 0 writes zeros.  The workspace holds the fp32 partial sums;
+ * launches that may run concurrently need a workspace each.
+ * Replaces autograd's F.linear backward for the gate's weight (xma/layers/moe/__init__.py:148,192).
+ */
+int64_t xma_router_weight_grad_workspace_bytes(int64_t T, int32_t E, int64_t H);
+int xma_router_weight_grad(const void* x, int64_t ldx, const void* d_logits, int64_t ldd, int dtype, int64_t T,
+                           int32_t E, int64_t H, void* dw, int64_t ldw, void* workspace, int64_t workspace_bytes,
+                           void* stream);
+
+/*
  * y = up * gate * sigmoid(gate), computed in fp32 (xma/functional/swiglu/__init__.py:34-43);
  * all operands [rows, cols] with independent row strides, so the two halves of a packed
  * tensor can be passed as views (xma/functional/swiglu_packed.py:48).

@@ -130,3 +130,46 @@ def test_topk_softmax_backward(dtype):
     ow.backward(dw)
     assert_close(lg.grad, lo.grad, TOL[dtype] * (1 if dtype == torch.float32 else 1), "d_logits")
     assert int((lg.grad != 0).sum(dim=-1).max()) <= k
+
+
+@pytest.mark.parametrize(
+    "T,E,H,dtype",
+    [
+        (8192, 8, 4096, torch.bfloat16),  # the benchmark layer's gate
+        (16384, 64, 2048, torch.bfloat16),  # fine-grained
+        (16384, 128, 2048, torch.bfloat16),  # skewed
+        (1000, 128, 520, torch.float16),  # ragged last stage, last column tile partly outside
+        (70, 256, 72, torch.bfloat16),
+        (1, 16, 8, torch.float16),
+        (0, 8, 64, torch.bfloat16),  # no tokens: zeros
+    ],
+)
+def test_router_weight_grad(T, E, H, dtype):
+    """dW = d_logits^T x against an fp32 matmul over the same 16-bit-valued operands (summation order and the final
+    rounding are the only differences), on row-strided views."""
+
+    from flash_model_architectures_amd import ops
+
+    from .helpers import GEMM_ELEM_TOL
+
+    g = torch.Generator().manual_seed(T + E + H)
+    x_full = torch.randn(T, H + 8, generator=g).to(dtype).cuda()
+    d_full = torch.randn(T, E + 8, generator=g).to(dtype).cuda()
+    x, d_logits = x_full[:, :H], d_full[:, :E]
+    assert ops.router_weight_grad_supported(x, d_logits)
+    dw = torch.full((E, H), float("nan"), dtype=dtype, device="cuda")
+    ops.router_weight_grad(x, d_logits, dw)
+    want = d_logits.float().t() @ x.float()
+    assert_close(dw, want, TOL[dtype], "router dW", elem_tol=GEMM_ELEM_TOL[dtype])
+    again = torch.empty_like(dw)
+    ops.router_weight_grad(x, d_logits, again)
+    assert torch.equal(dw, again)  # fixed summation order
+
+
+def test_router_weight_grad_falls_back_for_other_shapes():
+    from flash_model_architectures_amd import ops
+
+    x = torch.randn(64, 100, device="cuda", dtype=torch.bfloat16)
+    assert not ops.router_weight_grad_supported(x, torch.randn(64, 6, device="cuda", dtype=torch.bfloat16))  # E % 8
+    assert not ops.router_weight_grad_supported(x.float(), torch.randn(64, 8, device="cuda"))  # fp32
+    assert not ops.router_weight_grad_supported(x[:, 1:97], torch.randn(64, 8, device="cuda", dtype=torch.bfloat16))
