@@ -18,7 +18,7 @@ typedef __attribute__((ext_vector_type(4))) short short4_t;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 #define XMA_ROUTER_LDS_S4(p) ((__attribute__((address_space(3))) short4_t*)(p))
 
-constexpr int BT = 64;      // tokens per stage
+constexpr int BT = 128;     // tokens per stage
 constexpr int BH = 64;      // output columns per block: 4 waves x 16
 constexpr int THREADS = 256;
 constexpr int X_PITCH = BH * 2 + 16;  // bytes per token row of the x tile (padded: rows four apart fall into different banks)
