@@ -35,6 +35,7 @@ def test_header_declares_the_expected_entry_points():
         "xma_scatter_rows_ordered",
         "xma_combine_topk",
         "xma_gate_grad",
+        "xma_router_weight_grad",
         "xma_swiglu_forward",
         "xma_swiglu_backward",
         "xma_grouped_gemm",
@@ -77,6 +78,15 @@ def test_identification_and_error_channel():
     args.expert_offsets = ctypes.cast(off, ctypes.c_void_p)
     assert lib.xma_grouped_gemm(ctypes.byref(args), None) != 0 and "lda too small" in _native.last_error()
     assert lib.xma_grouped_gemm(None, None) != 0
+    out = (ctypes.c_uint16 * 64)()
+    rc = lib.xma_router_weight_grad(None, 8, None, 12, 2, 0, 12, 8, out, 8, None, 0, None)  # 12 experts: not a multiple of 8
+    assert rc != 0 and "multiple of 8" in _native.last_error()
+    rc = lib.xma_router_weight_grad(None, 8, None, 8, 0, 0, 8, 8, out, 8, None, 0, None)  # fp32
+    assert rc != 0 and "16-bit" in _native.last_error()
+    rc = lib.xma_router_weight_grad(out, 8, out, 8, 2, 64, 8, 8, out, 8, out, 16, None)  # workspace of 16 bytes
+    assert rc != 0 and "workspace too small" in _native.last_error()
+    assert lib.xma_router_weight_grad_workspace_bytes(0, 8, 4096) == 0
+    assert lib.xma_router_weight_grad_workspace_bytes(8192, 8, 4096) % (8 * 4096 * 4) == 0
     assert lib.xma_route_workspace_bytes(1 << 20, 256) == (1 << 20) // 1024 * 256 * 4
     assert lib.xma_grouped_gemm_workspace_bytes(8, 16384) >= (4 + 2 * (16384 // 128 + 8)) * 4
 
@@ -139,6 +149,7 @@ def test_moe_module_layout_and_state_dict():
                   activation_function=xma.swiglu_packed, is_glu=True, add_bias=False, std=0.02)
     assert moe.c_fc.weight.shape == (4, 48, 16) and moe.c_proj.weight.shape == (4, 16, 24)
     assert moe.gate.weight.shape == (4, 16) and moe.top_k == 2
+    assert isinstance(moe.gate, torch.nn.Linear) and moe.gate.bias is None  # nn.Linear in the reference (:148)
     keys = set(moe.state_dict().keys())
     assert keys == {"gate.weight", "c_fc.weight", "c_fc.N_array", "c_fc.K_array", "c_proj.weight",
                     "c_proj.N_array", "c_proj.K_array"}
