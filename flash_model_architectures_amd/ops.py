@@ -70,7 +70,8 @@ def exclusive_offsets(expert_offsets: torch.Tensor, E: int) -> torch.Tensor:
 #   * a buffer lives until release_workspaces() or the end of the process; a stream that has run a 16-bit grouped GEMM
 #     holds at least the 64 MiB split-K region;
 #   * ONE user at a time: the buffer serves, in turn, as tile tables and split-K region of a grouped GEMM, as the
-#     per-chunk histograms of route_build and as the inverted index of `ungroup`.  An operator must never need two of
+#     per-chunk histograms of route_build, as the partial sums of the router weight gradient and as the inverted index
+#     of `ungroup`.  An operator must never need two of
 #     these in one launch, and must not expect the contents to survive the next operator on the stream;
 #   * under stream capture (CUDA graphs) nothing is cached: a buffer allocated during capture belongs to the graph's
 #     private pool and must not be handed to later eager launches, so every captured call gets a buffer of its own
