@@ -762,7 +762,10 @@ int xma_continuous_count(const void* ids, int ids_is_i64, int64_t n, int32_t bin
         int copies = 2048 / bins;
         if (copies > 32) copies = 32;
         if (copies < 1) copies = 1;
-        const int per_block = 256 * 16;
+        // ids per block: every block ends with one global atomic per non-empty bin, all blocks onto the same few
+        // lines, so a stream of a million ids is faster over half as many blocks (6.0 against 7.2 us at 2^20 ids,
+        // 256 bins), while a short stream needs the blocks (98304 ids: 6.2 against 9.5 us)
+        const int per_block = n > ((int64_t)1 << 18) ? 256 * 32 : 256 * 16;
         int64_t blocks = ceil_div(n, per_block);
         if (blocks > 2048) blocks = 2048;
         const size_t lds = (size_t)bins * copies * sizeof(uint32_t);
