@@ -333,6 +333,47 @@ __global__ __launch_bounds__(256) void place_kernel(const IdT* __restrict__ ids,
         place_batch(v[j], begin + j * kWaveSize + lane, E, nbits, lane, next, sorted_ids, perm);
 }
 
+// The same placement by one block of four waves per unit, a quarter of the unit each (four batches in a row instead
+// of sixteen): every wave counts its quarter in LDS, thread e turns column e of the four rows into the first output
+// slot of expert e in each quarter, then the waves place their ids.  4 * E words of LDS: for E <= kQuarterMaxExperts.
+constexpr int kQuarterMaxExperts = 4096;
+template <typename IdT, typename OutT>
+__global__ __launch_bounds__(256) void place_quarters_kernel(const IdT* __restrict__ ids, int64_t n, int E, int nbits,
+                                                              const uint32_t* __restrict__ unit_prefix,
+                                                              const int32_t* __restrict__ offsets,
+                                                              OutT* __restrict__ sorted_ids, OutT* __restrict__ perm) {
+    extern __shared__ uint32_t lds_hist[];  // [4][E]: a quarter's histogram, then its next free output slots
+    const int wave = threadIdx.x / kWaveSize;
+    const int lane = lane_id();
+    const int64_t unit = blockIdx.x;
+    const int64_t begin = unit * kChunk + wave * kQuarter;
+    const int64_t end = begin + kQuarter < n ? begin + kQuarter : n;
+    int64_t v[kQuarterBatches];
+    load_chunk(ids, begin < n ? begin : n, end, lane, v);  // all -1 for a quarter past the end
+    for (int i = threadIdx.x; i < 4 * E; i += 256) lds_hist[i] = 0;
+    __syncthreads();
+    uint32_t* next = lds_hist + wave * E;
+#pragma unroll
+    for (int j = 0; j < kQuarterBatches; ++j)
+        if (v[j] >= 0 && v[j] < E) atomicAdd(&next[v[j]], 1u);
+    __syncthreads();
+    const uint32_t* row = unit_prefix + unit * E;
+    for (int e = threadIdx.x; e < E; e += 256) {
+        uint32_t slot = (uint32_t)offsets[e] + row[e];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t own = lds_hist[w * E + e];
+            lds_hist[w * E + e] = slot;
+            slot += own;
+        }
+    }
+    __syncthreads();
+    if (begin >= n) return;
+#pragma unroll
+    for (int j = 0; j < kQuarterBatches; ++j)
+        place_batch(v[j], begin + j * kWaveSize + lane, E, nbits, lane, next, sorted_ids, perm);
+}
+
 // Column sums of the table of per-unit histograms, by one block of 256 threads: total[e] += all units, before[e] +=
 // the units before `unit`.  A thread handles V adjacent experts (one 4 * V-byte load per unit) of the units r,
 // r + rows, ...; the number of thread columns is E / V rounded up to a power of two, so consecutive lanes read
@@ -846,22 +887,41 @@ static int route_build_launch(const void* ids, int ids_is_i64, int64_t n, int32_
 #undef XMA_SCAN_PLACE
         return check_launch("xma_route_build");
     }
+    // four launches: histograms, column scan over the units, scan over the experts, placement; a unit belongs to a
+    // block of four waves while four rows of E words fit in LDS, to one wave beyond
+    const bool quarters = E <= kQuarterMaxExperts;
     const int wpb = sort_waves_per_block(E);
     const unsigned blocks = (unsigned)ceil_div(units, wpb);
     const size_t lds = (size_t)wpb * E * sizeof(uint32_t);
-    if (ids_is_i64)
+    const size_t quarter_lds = (size_t)4 * E * sizeof(uint32_t);
+    if (quarters) {
+        if (ids_is_i64)
+            hipLaunchKernelGGL(block_hist_kernel<int64_t>, dim3((unsigned)units), dim3(256), quarter_lds, stream,
+                               (const int64_t*)ids, n, (int)E, unit_hist);
+        else
+            hipLaunchKernelGGL(block_hist_kernel<int32_t>, dim3((unsigned)units), dim3(256), quarter_lds, stream,
+                               (const int32_t*)ids, n, (int)E, unit_hist);
+    } else if (ids_is_i64) {
         hipLaunchKernelGGL(unit_hist_kernel<int64_t>, dim3(blocks), dim3(wpb * kWaveSize), lds, stream,
                            (const int64_t*)ids, n, (int)E, wpb, unit_hist);
-    else
+    } else {
         hipLaunchKernelGGL(unit_hist_kernel<int32_t>, dim3(blocks), dim3(wpb * kWaveSize), lds, stream,
                            (const int32_t*)ids, n, (int)E, wpb, unit_hist);
+    }
     hipLaunchKernelGGL(unit_scan_kernel, dim3((E + kWaveSize - 1) / kWaveSize), dim3(1024), 0, stream, unit_hist, units,
                        (int)E, counts);
     hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, stream, (const uint32_t*)counts, (int)E, offsets);
 #define XMA_PLACE(IdT, OutT)                                                                                       \
-    hipLaunchKernelGGL((place_kernel<IdT, OutT>), dim3(blocks), dim3(wpb * kWaveSize), lds, stream, (const IdT*)ids, \
-                       n, (int)E, nbits, wpb, (const uint32_t*)unit_hist, (const int32_t*)offsets,                 \
-                       (OutT*)sorted_ids, (OutT*)perm)
+    do {                                                                                                           \
+        if (quarters)                                                                                              \
+            hipLaunchKernelGGL((place_quarters_kernel<IdT, OutT>), dim3((unsigned)units), dim3(256), quarter_lds,  \
+                               stream, (const IdT*)ids, n, (int)E, nbits, (const uint32_t*)unit_hist,              \
+                               (const int32_t*)offsets, (OutT*)sorted_ids, (OutT*)perm);                           \
+        else                                                                                                       \
+            hipLaunchKernelGGL((place_kernel<IdT, OutT>), dim3(blocks), dim3(wpb * kWaveSize), lds, stream,         \
+                               (const IdT*)ids, n, (int)E, nbits, wpb, (const uint32_t*)unit_hist,                 \
+                               (const int32_t*)offsets, (OutT*)sorted_ids, (OutT*)perm);                           \
+    } while (0)
     if (ids_is_i64) {
         if (out_is_i64)
             XMA_PLACE(int64_t, int64_t);
