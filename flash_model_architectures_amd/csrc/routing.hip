@@ -350,6 +350,9 @@ __global__ __launch_bounds__(256) void place_quarters_kernel(const IdT* __restri
     const int64_t end = begin + kQuarter < n ? begin + kQuarter : n;
     int64_t v[kQuarterBatches];
     load_chunk(ids, begin < n ? begin : n, end, lane, v);  // all -1 for a quarter past the end
+    // where the unit's ids of expert e start: requested before the first barrier for the first 256 experts
+    const uint32_t* row = unit_prefix + unit * E;
+    const uint32_t first_start = (int)threadIdx.x < E ? (uint32_t)offsets[threadIdx.x] + row[threadIdx.x] : 0u;
     for (int i = threadIdx.x; i < 4 * E; i += 256) lds_hist[i] = 0;
     __syncthreads();
     uint32_t* next = lds_hist + wave * E;
@@ -357,9 +360,8 @@ __global__ __launch_bounds__(256) void place_quarters_kernel(const IdT* __restri
     for (int j = 0; j < kQuarterBatches; ++j)
         if (v[j] >= 0 && v[j] < E) atomicAdd(&next[v[j]], 1u);
     __syncthreads();
-    const uint32_t* row = unit_prefix + unit * E;
     for (int e = threadIdx.x; e < E; e += 256) {
-        uint32_t slot = (uint32_t)offsets[e] + row[e];
+        uint32_t slot = e < 256 ? first_start : (uint32_t)offsets[e] + row[e];
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             const uint32_t own = lds_hist[w * E + e];
@@ -890,6 +892,9 @@ static int route_build_launch(const void* ids, int ids_is_i64, int64_t n, int32_
     // four launches: histograms, column scan over the units, scan over the experts, placement; a unit belongs to a
     // block of four waves while four rows of E words fit in LDS, to one wave beyond
     const bool quarters = E <= kQuarterMaxExperts;
+    // (measured: 2^17 ids x 1024 experts 8.5 us against 19.2 us for the placement; 2^20 x 256 17.3 against 15.3 us,
+    // where a wave that walks 1024 ids writes four adjacent slots per expert)
+    const bool place_in_quarters = quarters && E > 256;
     const int wpb = sort_waves_per_block(E);
     const unsigned blocks = (unsigned)ceil_div(units, wpb);
     const size_t lds = (size_t)wpb * E * sizeof(uint32_t);
@@ -913,7 +918,7 @@ static int route_build_launch(const void* ids, int ids_is_i64, int64_t n, int32_
     hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, stream, (const uint32_t*)counts, (int)E, offsets);
 #define XMA_PLACE(IdT, OutT)                                                                                       \
     do {                                                                                                           \
-        if (quarters)                                                                                              \
+        if (place_in_quarters)                                                                                     \
             hipLaunchKernelGGL((place_quarters_kernel<IdT, OutT>), dim3((unsigned)units), dim3(256), quarter_lds,  \
                                stream, (const IdT*)ids, n, (int)E, nbits, (const uint32_t*)unit_hist,              \
                                (const int32_t*)offsets, (OutT*)sorted_ids, (OutT*)perm);                           \
