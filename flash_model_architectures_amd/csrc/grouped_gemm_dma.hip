@@ -389,7 +389,9 @@ struct Kernel {
     // every four 2.6 %; 16 slots with the reads spread out and the loads in even slots 1.4 %.  The kinds differ in
     // the best order of the reads: all A blocks, then all B blocks where both operands cost the same number of LDS
     // instructions (TN, MT), alternating where the transposed operand costs twice as many (NN).  One instruction
-    // per slot does not compile (the compiler runs out of scalar registers).
+    // per slot makes no difference where it compiles (NN: +-0.5 %); for TN and MT the compiler runs out of scalar
+    // registers ("illegal VGPR to SGPR copy"), and with the scalar operands of the loads forced through
+    // v_readfirstlane it spills thousands of vector registers.
     //
     // The tail tile of an expert's rows runs exactly the same instruction stream on zeros for the rows that do not
     // exist.  Skipping the missing 16-row blocks was measured and is a LOSS: the 32 work-groups an XCD runs at a
