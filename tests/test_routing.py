@@ -74,7 +74,9 @@ def test_route_full_size_invariants():
 
 
 @pytest.mark.parametrize("T,E,k", [(100, 8, 2), (1000, 64, 6), (1000, 128, 8), (64, 8, 1), (33, 300, 4), (7, 600, 8),
-                                   (5, 1000, 3), (3, 8, 8), (50, 2, 2)])
+                                   (5, 1000, 3), (3, 8, 8), (50, 2, 2),
+                                   # the remaining group widths of the kernel: 4, 32 and 64 lanes per token
+                                   (50, 16, 3), (40, 256, 8), (5, 512, 64), (131, 24, 1)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_topk_softmax_matches_oracle(T, E, k, dtype):
     g = torch.Generator().manual_seed(T * 7 + E + k)
