@@ -118,10 +118,11 @@ def test_topk_softmax_skewed_full_size():
     assert int((o.expert_frequency.to(torch.int64) == 0).sum()) >= 1  # ragged and empty groups are present
 
 
+@pytest.mark.parametrize("T,E,k", [(257, 64, 6), (100, 8, 2), (50, 16, 3), (40, 256, 8), (9, 512, 64), (64, 8, 1),
+                                   (7, 600, 8)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_topk_softmax_backward(dtype):
+def test_topk_softmax_backward(T, E, k, dtype):
     g = torch.Generator().manual_seed(5)
-    T, E, k = 257, 64, 6
     logits = torch.randn(T, E, generator=g).to(dtype)
     dw = torch.randn(T, k, generator=g).to(dtype)
     lg = logits.cuda().requires_grad_()
